@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 32
+ABI_VERSION = 33
 _lib = None
 _lock = threading.Lock()
 
@@ -37,9 +37,14 @@ _SIGNATURES = {
     "blm_moe_gate": [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_gla_scan": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_float, _c_void_p, _c_void_p,
                      _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                     _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
+                     _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_float, _c_int, _c_int, _c_void_p],
     "blm_qkv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
-                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                        _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                        _c_void_p],
+    "blm_scaled_add": [_c_void_p, _c_int, _c_int, _c_int] + [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int] * 4
+                      + [_c_void_p],
+    "blm_moe_route_grouped": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int,
+                              _c_void_p],
     "blm_sink_attn_mfma_supported": [_c_int, _c_int],
     "blm_sink_attn_mfma": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                            _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -1182,6 +1187,53 @@ def moe_gate(gate_up, weights, out, n_experts, expert_inner):
     return out
 
 
+def moe_route_grouped(logits, correction, n_experts, n_identity, groups, keep, top, weights):
+    """weights [T, E + 1] float32 from logits [T, >= E + n_identity] float32: scores are the softmax over all E + n_identity
+    logits; the choice goes by score + correction (None: the score) among the experts of the `keep` best of `groups`
+    equal groups of neighbours (a group's rank: its largest choice; groups <= 1: among all); the `top` chosen experts'
+    weights are their scores over the sum of the chosen scores.  Column e < E: expert e's weight or zero; column E: the
+    weights of the chosen ones among the last n_identity (experts that pass their input through), added up."""
+    _gpu(logits, correction, weights)
+    T = logits.shape[0]
+    _f32("logits", logits); _f32("weights", weights, T * (n_experts + 1))
+    if correction is not None:
+        _f32("correction", correction, n_experts + n_identity)
+    if logits.dim() != 2 or tuple(weights.shape) != (T, n_experts + 1):
+        raise KernelError("moe_route_grouped: logits [T, N], weights [T, E + 1]")
+    _call("blm_moe_route_grouped", logits.data_ptr(), logits.shape[1], _ptr(correction), int(n_experts), int(n_identity),
+          int(groups), int(keep), int(top), weights.data_ptr(), T, _stream())
+    return weights
+
+
+MAX_ADD_TERMS = 4
+
+
+def scaled_add(h, terms):
+    """h[t, c] += sum over terms (y, chan, row) of chan[c] * row[t] * y[t, c] in float32.  y: [T, D] in a kernel dtype or
+    float32 planes [P, T, D] (summed); chan: float32 [D] or None (one); row: float32 [T] (any stride) or None (one)."""
+    T, D = h.shape
+    _f32("h", h)
+    if not 1 <= len(terms) <= MAX_ADD_TERMS:
+        raise KernelError(f"scaled_add: one to {MAX_ADD_TERMS} terms, got {len(terms)}")
+    args = []
+    for y, chan, row in terms:
+        _gpu(y, chan, row)
+        planes, code = _planes("scaled_add: y", y, T, D)
+        if chan is not None:
+            _f32("chan", chan, D)
+        ld = 0
+        if row is not None:
+            if row.dtype != torch.float32 or row.dim() != 1 or row.shape[0] != T:
+                raise KernelError("scaled_add: a row coefficient is float32 [T]")
+            ld = row.stride(0) if T > 1 else 1
+            if ld < 1:
+                raise KernelError("scaled_add: a row coefficient's stride must be positive")
+        args += [y.data_ptr(), code, planes, _ptr(chan), _ptr(row), ld]
+    args += [0, 0, 0, 0, 0, 0] * (MAX_ADD_TERMS - len(terms))
+    _call("blm_scaled_add", h.data_ptr(), T, D, len(terms), *args, _stream())
+    return h
+
+
 def gla_segments(step, H, dv, compute_units=256):
     """(segments, tokens per segment) into which gla_scan cuts the sequences of a step: prompts are walked by several
     wavefronts at once, each over a stretch of at least 64 tokens (a multiple of 8), as many as give every compute
@@ -1196,19 +1248,38 @@ def gla_segments(step, H, dv, compute_units=256):
     return -(-step.max_new // seg_len), seg_len
 
 
-def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, step, H, dk, dv, segments=None):
+GATE_MODES = {"sigmoid": 1, "silu": 2}
+
+
+def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, step, H, dk, dv, segments=None,
+             fixed_decay=None, activation=None, q_scale=None, norm_all=False, gate="silu"):
     """Gated linear attention over proj [T, >= 2 H dk + 2 H dv]: queries, keys, values, output-gate logits;
     decay_in [T, H dk]: the decays' logits before their bias.  state float32 [slots, H, dk, dv] is read and left
     updated; o_raw: zeroed float32 [T, H * dv]; out [T, H * dv] in proj's dtype.  segments: (count, tokens each) as
-    gla_segments gives them (the default), or (1, 0) for one walk per sequence."""
-    _gpu(proj, decay_in, decay_bias, norm_w, state, o_raw, out)
+    gla_segments gives them (the default), or (1, 0) for one walk per sequence.
+    The same recurrence with other surroundings: fixed_decay (float32 [H * dk]): the decays of every token, in place of
+    decay_in, decay_bias and tau (which are then None); activation "silu": on queries, keys and values; q_scale: the
+    queries' factor (default dk^-1/2); norm_all: one root mean square over all heads' lanes, norm_w [H * dv] (default:
+    per head, norm_w [dv]); gate: "silu" or "sigmoid" of the output gate's logits."""
+    _gpu(proj, decay_in, decay_bias, norm_w, state, o_raw, out, fixed_decay)
     T = proj.shape[0]
-    _f32("o_raw", o_raw, T * H * dv); _f32("decay_bias", decay_bias, H * dk); _f32("norm_w", norm_w, dv); _f32("state", state)
-    _contig("decay_in", decay_in); _contig("out", out)
-    gates = torch.empty(T, H * dk, dtype=torch.float32, device=proj.device)
-    if proj.stride(1) != 1 or out.dtype != proj.dtype or decay_in.dtype != proj.dtype or tuple(out.shape) != (T, H * dv) \
-            or tuple(decay_in.shape) != (T, H * dk) or tuple(state.shape[1:]) != (H, dk, dv):
+    _f32("o_raw", o_raw, T * H * dv); _f32("norm_w", norm_w, H * dv if norm_all else dv); _f32("state", state)
+    _contig("out", out)
+    if activation not in (None, "silu") or gate not in GATE_MODES:
+        raise KernelError(f"gla_scan: activation {activation!r} or gate {gate!r} unknown")
+    if proj.stride(1) != 1 or out.dtype != proj.dtype or tuple(out.shape) != (T, H * dv) or tuple(state.shape[1:]) != (H, dk, dv) \
+            or proj.shape[1] < 2 * H * dk + 2 * H * dv or T != step.n_tokens:
         raise KernelError("gla_scan: shapes do not fit")
+    gates = None
+    if fixed_decay is not None:
+        _f32("fixed_decay", fixed_decay, H * dk)
+        if decay_in is not None or decay_bias is not None:
+            raise KernelError("gla_scan: fixed decays come without decay logits")
+    else:
+        _f32("decay_bias", decay_bias, H * dk); _contig("decay_in", decay_in)
+        if decay_in.dtype != proj.dtype or tuple(decay_in.shape) != (T, H * dk):
+            raise KernelError("gla_scan: shapes do not fit")
+        gates = torch.empty(T, H * dk, dtype=torch.float32, device=proj.device)
     n_seg, seg_len = segments if segments is not None else gla_segments(step, H, dv)
     seg_end = seg_start = seg_decay = q_tilde = None
     if n_seg > 1:
@@ -1217,23 +1288,29 @@ def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, st
         seg_start = torch.empty_like(seg_end)
         seg_decay = torch.empty(B, n_seg, H, dk, dtype=torch.float32, device=proj.device)
         q_tilde = torch.empty(T, H, dk, dtype=torch.float32, device=proj.device)
-    _call("blm_gla_scan", proj.data_ptr(), _code(proj), proj.stride(0), decay_in.data_ptr(), decay_bias.data_ptr(), float(tau),
-          norm_w.data_ptr(), float(eps), state.data_ptr(), gates.data_ptr(), o_raw.data_ptr(), out.data_ptr(),
-          step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, step.n_seqs, H, dk, dv, step.max_new, n_seg, seg_len,
-          _ptr(seg_end), _ptr(seg_start), _ptr(seg_decay), _ptr(q_tilde), _stream())
+    _call("blm_gla_scan", proj.data_ptr(), _code(proj), proj.stride(0), _ptr(decay_in), _ptr(decay_bias),
+          float(tau) if tau is not None else 0.0, norm_w.data_ptr(), float(eps), state.data_ptr(), _ptr(gates), o_raw.data_ptr(),
+          out.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, step.n_seqs, H, dk, dv, step.max_new, n_seg,
+          seg_len, _ptr(seg_end), _ptr(seg_start), _ptr(seg_decay), _ptr(q_tilde), _ptr(fixed_decay),
+          1 if activation == "silu" else 0, float(q_scale) if q_scale is not None else 0.0, 1 if norm_all else 0,
+          GATE_MODES[gate], _stream())
     return out
 
 
-def qkv_prepare(qkv, bias, cos_sin, rot, step, block_table, kcache, vcache, page_size, H, G, dk, dv, write_kv=True):
+def qkv_prepare(qkv, bias, cos_sin, rot, step, block_table, kcache, vcache, page_size, H, G, dk, dv, write_kv=True,
+                adjacent=False, values_are_keys=False):
     """Bias, rotation of the first `rot` lanes of every query and key head by the token's position (lane i with
-    lane i + rot/2; cos_sin float32 [positions, >= rot/2, 2] rows of exactly rot/2 pairs), queries in place, rotated
-    keys and values into the pages (key pages [pages, G, page, dk], value pages [pages, G, dv, page]).  write_kv
-    False: qkv holds queries only and nothing is stored."""
+    lane i + rot/2, or with adjacent lanes 2i and 2i + 1; cos_sin float32 [positions, >= rot/2, 2] rows of exactly
+    rot/2 pairs), queries in place, rotated keys and values into the pages (key pages [pages, G, page, dk], value pages
+    [pages, G, dv, page]).  write_kv False: qkv holds queries only and nothing is stored.  values_are_keys: the rows
+    hold no values; a token's values are its keys as projected, before the rotation (dv = dk)."""
     _gpu(qkv, bias, cos_sin, block_table, kcache, vcache)
     T = qkv.shape[0]
     if qkv.stride(1) != 1:
         raise KernelError("qkv_prepare: rows must be contiguous")
-    need = H * dk + (G * (dk + dv) if write_kv else 0)
+    if values_are_keys and dv != dk:
+        raise KernelError("qkv_prepare: values that are the keys have the keys' head size")
+    need = H * dk + (G * (dk + (0 if values_are_keys else dv)) if write_kv else 0)
     if qkv.shape[1] < need or T != step.n_tokens:
         raise KernelError(f"qkv_prepare: rows of {qkv.shape[1]}, needs {need}")
     if bias is not None:
@@ -1250,7 +1327,7 @@ def qkv_prepare(qkv, bias, cos_sin, rot, step, block_table, kcache, vcache, page
     _call("blm_qkv_prepare", qkv.data_ptr(), _code(qkv), qkv.stride(0), _ptr(bias), _ptr(cos_sin) if rot else 0, rot,
           step.positions.data_ptr(), step.token_seq.data_ptr(), _ptr(block_table) if write_kv else 0,
           block_table.shape[1] if write_kv else 0, _ptr(kcache) if write_kv else 0, _ptr(vcache) if write_kv else 0,
-          page_size, T, H, G, dk, dv, 1 if write_kv else 0, _stream())
+          page_size, T, H, G, dk, dv, 1 if write_kv else 0, 1 if adjacent else 0, 1 if values_are_keys else 0, _stream())
     return qkv
 
 

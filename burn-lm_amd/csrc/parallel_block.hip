@@ -432,3 +432,160 @@ extern "C" int blm_moe_gate(const void* gate_up, const float* weights, void* out
   BLM_LAUNCH_CHECK("moe_gate");
   return 0;
 }
+
+// ---------------------------------------------------------------------------------------
+// Several sublayers' results into the residual at once, each with a coefficient per channel and (optionally) per
+// token:  h[t][c] += sum_i chan_i[c] * row_i[t] * sum_p y_i[p][t][c]  in float.  A term's y is [T][D] in any kernel
+// dtype or float planes [P][T][D]; chan_i (float [D]) or row_i (float, row t at row_i[t * row_ld_i]) may be null
+// (a factor of one).  This is how a layer with layer scale and a residual multiplier adds mixer and feed-forward,
+// and how a sublayer that passes its input through (an identity expert) adds weight * input.
+// ---------------------------------------------------------------------------------------
+#define PB_MAX_TERMS 4
+struct PbTerms {
+  const void* y[PB_MAX_TERMS];
+  const float* chan[PB_MAX_TERMS];
+  const float* row[PB_MAX_TERMS];
+  int row_ld[PB_MAX_TERMS];
+  int planes[PB_MAX_TERMS];
+  int dtype[PB_MAX_TERMS];
+};
+
+__global__ void scaled_add_kernel(float* __restrict__ h, PbTerms tm, int n_terms, long long n, int D) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const long long t = e / D;
+    const int c = (int)(e - t * D);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < PB_MAX_TERMS; ++i) {
+      if (i < n_terms) {
+        float y = 0.f;
+        if (tm.dtype[i] == BLM_F32) {
+          const float* p = (const float*)tm.y[i];
+          for (int k = 0; k < tm.planes[i]; ++k) y += p[(size_t)k * n + e];
+        } else {
+          y = to_float(((const bf16*)tm.y[i])[e]);
+        }
+        float f = tm.chan[i] ? tm.chan[i][c] : 1.0f;
+        if (tm.row[i]) f *= tm.row[i][(size_t)t * tm.row_ld[i]];
+        sum = fmaf(f, y, sum);
+      }
+    }
+    h[e] += sum;
+  }
+}
+
+extern "C" int blm_scaled_add(float* h, int T, int D, int n_terms,
+                              const void* y0, int dtype0, int planes0, const float* chan0, const float* row0, int row_ld0,
+                              const void* y1, int dtype1, int planes1, const float* chan1, const float* row1, int row_ld1,
+                              const void* y2, int dtype2, int planes2, const float* chan2, const float* row2, int row_ld2,
+                              const void* y3, int dtype3, int planes3, const float* chan3, const float* row3, int row_ld3,
+                              hipStream_t stream) {
+  BLM_REQUIRE(h && T > 0 && D > 0 && n_terms >= 1 && n_terms <= PB_MAX_TERMS, "scaled_add: bad sizes T=%d D=%d terms=%d", T, D, n_terms);
+  PbTerms tm;
+  const void* ys[PB_MAX_TERMS] = {y0, y1, y2, y3};
+  const float* chans[PB_MAX_TERMS] = {chan0, chan1, chan2, chan3};
+  const float* rows[PB_MAX_TERMS] = {row0, row1, row2, row3};
+  const int lds[PB_MAX_TERMS] = {row_ld0, row_ld1, row_ld2, row_ld3};
+  const int planes[PB_MAX_TERMS] = {planes0, planes1, planes2, planes3};
+  const int dtypes[PB_MAX_TERMS] = {dtype0, dtype1, dtype2, dtype3};
+  for (int i = 0; i < PB_MAX_TERMS; ++i) {
+    const bool used = i < n_terms;
+    BLM_REQUIRE(!used || (ys[i] && planes[i] >= 1 && (dtypes[i] == BLM_F32 || (dtypes[i] == BLM_BF16 && planes[i] == 1)) &&
+                          (!rows[i] || lds[i] >= 1)),
+                "scaled_add: term %d is not float planes or one bfloat16 plane", i);
+    tm.y[i] = used ? ys[i] : nullptr;
+    tm.chan[i] = used ? chans[i] : nullptr;
+    tm.row[i] = used ? rows[i] : nullptr;
+    tm.row_ld[i] = used ? lds[i] : 0;
+    tm.planes[i] = used ? planes[i] : 0;
+    tm.dtype[i] = used ? dtypes[i] : BLM_F32;
+  }
+  const long long n = (long long)T * D;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  hipLaunchKernelGGL(scaled_add_kernel, dim3(blocks), dim3(256), 0, stream, h, tm, n_terms, n, D);
+  BLM_LAUNCH_CHECK("scaled_add");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// Routing by scores with a correction, limited to the best groups.  logits [T][ld] float: N = E + n_identity router
+// logits (the last n_identity belong to experts that pass their input through).  s = softmax(logits) over all N;
+// choice = s + correction (null: none).  The N experts form `groups` equal groups of neighbours; a group's score is its
+// largest choice; only experts of the `keep` best groups can be chosen (groups <= 1: all can).  The `top` largest
+// choices are taken (the lower index wins a tie); their weights are s (without the correction) over the sum of the
+// chosen s (+ 1e-20).  weights [T][E + 1] float: a real expert's weight or 0, and at E the sum of the weights of the
+// chosen pass-through experts.
+// ---------------------------------------------------------------------------------------
+#define PB_MAX_ROUTED 256
+__global__ void moe_route_grouped_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction,
+                                         int E, int n_identity, int groups, int keep, int top, float* __restrict__ weights,
+                                         int T) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const int N = E + n_identity;
+  const float* z = logits + (size_t)t * ld;
+  float* w = weights + (size_t)t * (E + 1);
+  float largest = z[0];
+  for (int e = 1; e < N; ++e) largest = fmaxf(largest, z[e]);
+  float denom = 0.f;
+  for (int e = 0; e < N; ++e) denom += expf(z[e] - largest);
+  const float inv = 1.0f / denom;
+  auto score = [&](int e) { return expf(z[e] - largest) * inv; };
+  auto choice = [&](int e) { return score(e) + (correction ? correction[e] : 0.f); };
+  // the groups that stay: `keep` times the best group not yet taken (a bit per group)
+  unsigned long long kept[PB_MAX_ROUTED / 64] = {0ull, 0ull, 0ull, 0ull};
+  const int per = groups > 1 ? N / groups : N;
+  if (groups > 1) {
+    for (int k = 0; k < keep; ++k) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int g = 0; g < groups; ++g) {
+        if (kept[g >> 6] >> (g & 63) & 1ull) continue;
+        float gv = -INFINITY;
+        for (int e = g * per; e < (g + 1) * per; ++e) gv = fmaxf(gv, choice(e));
+        if (best < 0 || gv > bv) { best = g; bv = gv; }
+      }
+      kept[best >> 6] |= 1ull << (best & 63);
+    }
+  }
+  for (int e = 0; e <= E; ++e) w[e] = 0.f;
+  int chosen[PB_MAX_TOP];
+  float val[PB_MAX_TOP];
+  float sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < N; ++e) {
+      if (groups > 1) {
+        const int g = e / per;
+        if (!(kept[g >> 6] >> (g & 63) & 1ull)) continue;
+      }
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken |= chosen[j] == e;
+      if (taken) continue;
+      const float v = choice(e);
+      if (best < 0 || v > bv) { best = e; bv = v; }
+    }
+    chosen[k] = best;
+    val[k] = score(best);
+    sum += val[k];
+  }
+  const float norm = 1.0f / (sum + 1e-20f);
+  for (int k = 0; k < top; ++k) w[chosen[k] < E ? chosen[k] : E] += val[k] * norm;
+}
+
+extern "C" int blm_moe_route_grouped(const float* logits, int ld, const float* correction, int E, int n_identity, int groups,
+                                     int keep, int top, float* weights, int T, hipStream_t stream) {
+  const int N = E + n_identity;
+  BLM_REQUIRE(T > 0 && E >= 0 && n_identity >= 0 && N >= 1 && N <= PB_MAX_ROUTED && ld >= N && top >= 1 && top <= PB_MAX_TOP,
+              "moe_route_grouped: bad sizes T=%d experts=%d+%d (at most %d) top=%d (at most %d)", T, E, n_identity,
+              PB_MAX_ROUTED, top, PB_MAX_TOP);
+  BLM_REQUIRE(groups <= 1 || (N % groups == 0 && keep >= 1 && keep <= groups), "moe_route_grouped: %d experts in %d groups, %d kept",
+              N, groups, keep);
+  BLM_REQUIRE(top <= (groups > 1 ? keep * (N / groups) : N), "moe_route_grouped: top=%d is more than the kept groups hold", top);
+  hipLaunchKernelGGL(moe_route_grouped_kernel, dim3((T + 127) / 128), dim3(128), 0, stream, logits, ld, correction, E,
+                     n_identity, groups, keep, top, weights, T);
+  BLM_LAUNCH_CHECK("moe_route_grouped");
+  return 0;
+}

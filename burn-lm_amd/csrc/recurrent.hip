@@ -584,7 +584,7 @@ __global__ void gla_gates_kernel(const TA* __restrict__ decay_in, const float* _
 // gla_apply_kernel adds the first term to the results.  Decays are at most one, so the products cannot overflow.
 template <typename TA, int ROWS, int LPC, bool SEG, int CH>
 __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
-    gla_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ gates, float q_scale,
+    gla_scan_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ gates, int gates_ld, int act, float q_scale,
                     float* __restrict__ state, float* __restrict__ o_raw, const int* __restrict__ cu_seqlens,
                     const int* __restrict__ seq_slots, int H, int dk, int dv, int col_groups, long long n_items,
                     int n_seg, int seg_len, float* __restrict__ seg_end, float* __restrict__ seg_decay,
@@ -627,17 +627,19 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
       if (tc + tt < t1) {
         const int t = tc + tt;
         const TA* row = proj + (size_t)t * ld;
-        const float* gr = gates + (size_t)t * H * dk;
+        const float* gr = gates + (size_t)t * gates_ld;
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
           const int i = lane + k * BLM_WAVE;
           if (i < dk) {
             raw_d[tt][k] = gr[h * dk + i];
-            raw_k[tt][k] = to_float(row[(size_t)H * dk + h * dk + i]);
-            raw_q[tt][k] = to_float(row[h * dk + i]) * q_scale;
+            const float kx = to_float(row[(size_t)H * dk + h * dk + i]), qx = to_float(row[h * dk + i]);
+            raw_k[tt][k] = act ? blm_silu(kx) : kx;
+            raw_q[tt][k] = (act ? blm_silu(qx) : qx) * q_scale;
           }
         }
         v_in[tt] = own ? to_float(row[(size_t)2 * H * dk + h * dv + col]) : 0.f;
+        if (act) v_in[tt] = blm_silu(v_in[tt]);
       }
     }
   };
@@ -784,19 +786,28 @@ __global__ void __launch_bounds__(BLM_WAVE)
 
 // n_seg > 1 (only where the sequences bring many tokens each, T > 4 B): seg_len a multiple of 8 with n_seg * seg_len >= the
 // most tokens of a sequence; seg_end and seg_start [B][n_seg][H][dk][dv], seg_decay [B][n_seg][H][dk], q_tilde [T][H][dk].
+// Variants of the same recurrence, for mixers that differ in what surrounds it:
+//   fixed_decay [H*dk] float (not null): every token's decays, instead of decay_in, decay_bias and tau (a decay per head that
+//     is a constant of the model; gates is then not used);
+//   act_mode 1: SiLU on the queries, keys and values as they are read;  q_scale: the queries' factor (<= 0: dk^-1/2);
+//   norm_all 1: the root mean square is taken over all heads' value lanes together and norm_w is [H*dv];
+//   gate_mode: 1 sigmoid, 2 SiLU of the output gate's logits.
 extern "C" int blm_gla_scan(const void* proj, int dtype, int ld, const void* decay_in, const float* decay_bias, float tau,
                             const float* norm_w, float eps, float* state, float* gates, float* o_raw, void* out,
                             const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int dk, int dv, int max_new,
                             int n_seg, int seg_len, float* seg_end, float* seg_start, float* seg_decay, float* q_tilde,
+                            const float* fixed_decay, int act_mode, float q_scale_in, int norm_all, int gate_mode,
                             hipStream_t stream) {
-  BLM_REQUIRE(T > 0 && B > 0 && H > 0 && tau > 0.f, "gla_scan: bad sizes T=%d B=%d H=%d tau=%g", T, B, H, (double)tau);
+  BLM_REQUIRE(T > 0 && B > 0 && H > 0 && (fixed_decay || tau > 0.f), "gla_scan: bad sizes T=%d B=%d H=%d tau=%g", T, B, H, (double)tau);
   BLM_REQUIRE(dk >= 1 && dk <= SCAN_MAX_DK && dv >= 1, "gla_scan: %d key channels per head are not supported (up to %d)", dk, SCAN_MAX_DK);
   BLM_REQUIRE(ld >= 2 * H * dk + 2 * H * dv, "gla_scan: rows of %d are too short", ld);
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "gla_scan: unsupported dtype %d", dtype);
   BLM_REQUIRE(n_seg >= 1 && (n_seg == 1 || (T > 4 * B && seg_len >= 8 && seg_len % 8 == 0 && (long long)n_seg * seg_len >= max_new &&
                                             dv <= BLM_WAVE * GLA_APPLY_CPL && seg_end && seg_start && seg_decay && q_tilde)),
               "gla_scan: %d segments of %d tokens do not fit this step", n_seg, seg_len);
-  {
+  BLM_REQUIRE((act_mode == 0 || act_mode == 1) && (gate_mode == 1 || gate_mode == 2) && (fixed_decay || (decay_in && decay_bias && gates)),
+              "gla_scan: unknown activation %d or gate %d, or no decays", act_mode, gate_mode);
+  if (!fixed_decay) {
     const long long n = (long long)T * H * dk;
     const unsigned gblocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
     if (dtype == BLM_F32)
@@ -805,17 +816,19 @@ extern "C" int blm_gla_scan(const void* proj, int dtype, int ld, const void* dec
       hipLaunchKernelGGL(gla_gates_kernel<bf16>, dim3(gblocks), dim3(256), 0, stream, (const bf16*)decay_in, decay_bias, 1.0f / tau, gates, n, H * dk);
     BLM_LAUNCH_CHECK("gla_gates");
   }
-  const float q_scale = 1.0f / sqrtf((float)dk);
+  const float q_scale = q_scale_in > 0.f ? q_scale_in : 1.0f / sqrtf((float)dk);
+  const float* decays = fixed_decay ? fixed_decay : gates;
+  const int decays_ld = fixed_decay ? 0 : H * dk;
 #define BLM_GLA_RUN(ROWS, LPC, SEG, NSEG, CH)                                                                             \
   const int col_groups = (dv + 64 / LPC - 1) / (64 / LPC);                                                                \
   const long long items = (long long)B * NSEG * H * col_groups;                                                           \
   const ScanLaunch sl = scan_launch(ROWS, LPC, 3, items, CH);                                                             \
   if (dtype == BLM_F32)                                                                                                   \
-    hipLaunchKernelGGL((gla_scan_kernel<float, ROWS, LPC, SEG, CH>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, gates, \
+    hipLaunchKernelGGL((gla_scan_kernel<float, ROWS, LPC, SEG, CH>), sl.grid, sl.block, sl.smem, stream, (const float*)proj, ld, decays, decays_ld, act_mode, \
                        q_scale, state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items, n_seg, seg_len, seg_end, \
                        seg_decay, q_tilde);                                                                               \
   else                                                                                                                    \
-    hipLaunchKernelGGL((gla_scan_kernel<bf16, ROWS, LPC, SEG, CH>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, gates,   \
+    hipLaunchKernelGGL((gla_scan_kernel<bf16, ROWS, LPC, SEG, CH>), sl.grid, sl.block, sl.smem, stream, (const bf16*)proj, ld, decays, decays_ld, act_mode,   \
                        q_scale, state, o_raw, cu_seqlens, seq_slots, H, dk, dv, col_groups, items, n_seg, seg_len, seg_end, \
                        seg_decay, q_tilde)
   // segments: many wavefronts at once, each waiting for its own chain of dependent instructions; chunks of four tokens halve
@@ -847,5 +860,6 @@ extern "C" int blm_gla_scan(const void* proj, int dtype, int ld, const void* dec
     BLM_LAUNCH_CHECK("gla_apply");
   }
   const char* gate = (const char*)proj + (size_t)(2 * H * dk + H * dv) * (dtype == BLM_F32 ? 4 : 2);
-  return launch_head_norm(o_raw, norm_w, gate, ld, 2, H, out, dtype, (long long)T * H, dv, eps, stream);
+  if (norm_all) return launch_head_norm(o_raw, norm_w, gate, ld, gate_mode, 1, out, dtype, (long long)T, H * dv, eps, stream);
+  return launch_head_norm(o_raw, norm_w, gate, ld, gate_mode, H, out, dtype, (long long)T * H, dv, eps, stream);
 }

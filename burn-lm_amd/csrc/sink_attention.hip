@@ -19,14 +19,16 @@
 
 // ---------------------------------------------------------------------------------------
 // qkv [T][ld]: queries at column 0 (H * dk), then (if keys are written) keys (G * dk) and values (G * dv).
-// bias [H*dk (+ G*dk + G*dv)] float or null.  cos_sin [positions][rot/2][2] float.
+// bias [H*dk (+ G*dk + G*dv)] float or null.  cos_sin [positions][rot/2][2] float.  adjacent: pair i of the turning
+// lanes is (2i, 2i + 1) instead of (i, i + rot/2).  values_are_keys (dv = dk): there are no value columns; a token's
+// values are its keys as projected (with their bias), before the rotation.
 // ---------------------------------------------------------------------------------------
 template <typename TA>
 __global__ void qkv_prepare_kernel(TA* __restrict__ qkv, int ld, const float* __restrict__ bias,
                                    const float* __restrict__ cos_sin, int rot, const int* __restrict__ positions,
                                    const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_width,
                                    TA* __restrict__ kcache, TA* __restrict__ vcache, int page_size, int H, int G, int dk,
-                                   int dv, int write_kv) {
+                                   int dv, int write_kv, int adjacent, int values_are_keys) {
   const int t = blockIdx.x;
   const int b = token_seq[t];
   if (b < 0) return;
@@ -47,12 +49,13 @@ __global__ void qkv_prepare_kernel(TA* __restrict__ qkv, int ld, const float* __
     const int col = head * dk;
     TA* krow = head >= H ? kcache + (((size_t)page * G + (head - H)) * page_size + in_page) * dk : nullptr;
     if (i < half) {
-      float u = to_float(row[col + i]), v = to_float(row[col + i + half]);
-      if (bias) { u += bias[col + i]; v += bias[col + i + half]; }
+      const int la = adjacent ? 2 * i : i, lb = adjacent ? 2 * i + 1 : i + half;
+      float u = to_float(row[col + la]), v = to_float(row[col + lb]);
+      if (bias) { u += bias[col + la]; v += bias[col + lb]; }
       const float c = cs[2 * i], s = cs[2 * i + 1];
       const float ru = u * c - v * s, rv = v * c + u * s;
-      if (krow) { krow[i] = from_float<TA>(ru); krow[i + half] = from_float<TA>(rv); }
-      else { row[col + i] = from_float<TA>(ru); row[col + i + half] = from_float<TA>(rv); }
+      if (krow) { krow[la] = from_float<TA>(ru); krow[lb] = from_float<TA>(rv); }
+      else { row[col + la] = from_float<TA>(ru); row[col + lb] = from_float<TA>(rv); }
     } else {
       const int lane = rot + (i - half);
       float u = to_float(row[col + lane]);
@@ -62,7 +65,8 @@ __global__ void qkv_prepare_kernel(TA* __restrict__ qkv, int ld, const float* __
     }
   }
   if (write_kv) {
-    const int v0 = (H + G) * dk;
+    // the keys' columns of the row still hold what was projected (rotated keys went to the pages only)
+    const int v0 = values_are_keys ? H * dk : (H + G) * dk;
     for (int e = threadIdx.x; e < G * dv; e += blockDim.x) {
       float u = to_float(row[v0 + e]);
       if (bias) u += bias[v0 + e];
@@ -75,18 +79,19 @@ __global__ void qkv_prepare_kernel(TA* __restrict__ qkv, int ld, const float* __
 extern "C" int blm_qkv_prepare(void* qkv, int dtype, int ld, const float* bias, const float* cos_sin, int rot,
                                const int* positions, const int* token_seq, const int* block_table, int table_width,
                                void* kcache, void* vcache, int page_size, int T, int H, int G, int dk, int dv, int write_kv,
-                               hipStream_t stream) {
+                               int adjacent, int values_are_keys, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && H > 0 && G > 0 && dk > 0 && dv > 0, "qkv_prepare: bad sizes T=%d H=%d G=%d dk=%d dv=%d", T, H, G, dk, dv);
   BLM_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dk, "qkv_prepare: %d turning lanes of %d (even, at most the head size)", rot, dk);
-  BLM_REQUIRE(ld >= H * dk + (write_kv ? G * (dk + dv) : 0), "qkv_prepare: rows of %d are too short", ld);
+  BLM_REQUIRE(!values_are_keys || dv == dk, "qkv_prepare: values that are the keys have the keys' head size, not %d", dv);
+  BLM_REQUIRE(ld >= H * dk + (write_kv ? G * (dk + (values_are_keys ? 0 : dv)) : 0), "qkv_prepare: rows of %d are too short", ld);
   BLM_REQUIRE(!write_kv || (kcache && vcache && block_table && page_size > 0 && table_width > 0), "qkv_prepare: the pages are missing");
   BLM_REQUIRE(rot == 0 || cos_sin, "qkv_prepare: the table of angles is missing");
   if (dtype == BLM_F32)
     hipLaunchKernelGGL(qkv_prepare_kernel<float>, dim3(T), dim3(256), 0, stream, (float*)qkv, ld, bias, cos_sin, rot, positions,
-                       token_seq, block_table, table_width, (float*)kcache, (float*)vcache, page_size, H, G, dk, dv, write_kv);
+                       token_seq, block_table, table_width, (float*)kcache, (float*)vcache, page_size, H, G, dk, dv, write_kv, adjacent, values_are_keys);
   else if (dtype == BLM_BF16)
     hipLaunchKernelGGL(qkv_prepare_kernel<bf16>, dim3(T), dim3(256), 0, stream, (bf16*)qkv, ld, bias, cos_sin, rot, positions,
-                       token_seq, block_table, table_width, (bf16*)kcache, (bf16*)vcache, page_size, H, G, dk, dv, write_kv);
+                       token_seq, block_table, table_width, (bf16*)kcache, (bf16*)vcache, page_size, H, G, dk, dv, write_kv, adjacent, values_are_keys);
   else
     return blm_fail("qkv_prepare: unsupported dtype %d", dtype);
   BLM_LAUNCH_CHECK("qkv_prepare");

@@ -11,11 +11,14 @@ from .embedding import Embedding, LMHead
 from .gla import GatedLinearAttention
 from .hgrn2 import HGRN2
 from .latent_attention import LatentAttention
+from .lightning import LightningAttention
+from .mixer_pair import MixerPair
 from .norm_layer import LayerNorm
 from .norm_rms import RMSNorm
-from .parallel import CausalConvInput, ParallelBlock, ParallelMixerBlock, TokenSide
+from .parallel import (CausalConvInput, LayerScale, ParallelBlock, ParallelMixerBlock, ScaledParallelBlock,
+                       ScaledParallelMixerBlock, TokenSide)
 from .rope import RotaryEncoding
-from .routed_experts import RoutedExperts
+from .routed_experts import GroupedRoutedExperts, RoutedExperts
 from .sink_attention import SinkAttention
 from .streams import HyperBlock, HyperConnection, HyperMixerBlock
 from .swiglu import SwiGLU
@@ -43,3 +46,9 @@ registry.register_part("connection", "causal_conv", CausalConvInput)
 registry.register_part("connection", "token_side", TokenSide)
 registry.register_part("block", "parallel", ParallelBlock)
 registry.register_part("block", "parallel_mixer_only", ParallelMixerBlock)
+registry.register_part("mixer", "lightning_attention", LightningAttention)
+registry.register_part("mixer", "mixer_pair", MixerPair)
+registry.register_part("feed_forward", "grouped_experts", GroupedRoutedExperts)
+registry.register_part("connection", "layer_scale", LayerScale)
+registry.register_part("block", "parallel_scaled", ScaledParallelBlock)
+registry.register_part("block", "parallel_scaled_mixer_only", ScaledParallelMixerBlock)

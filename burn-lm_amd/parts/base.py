@@ -16,7 +16,8 @@ Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the act
 * ``Mixer.cache_need() -> KVNeed | StateNeed | None`` and
   ``Mixer.forward(x, step, view) -> delta``; ``view`` is what the cache holds for this place
   in the layer order (``KVView``, ``StateView`` or ``None``).
-* ``FeedForward.forward(x, step) -> delta``.
+* ``FeedForward.forward(x, step) -> delta``.  Both also have ``forward_terms(...) -> [Term]``: the same result as
+  summands ``scale * row[t] * y[t]`` for a block that adds them to the residual itself with further coefficients.
 * ``PositionEncoding.prepare(n_positions, rt)``, ``for_projection(w_q, w_k, heads, kv_heads)`` (the
   encoding may re-order the projections' rows when they are bound) and, for encodings that act on queries and keys,
   ``encode_and_store(qkv, step, view, heads, kv_heads, head_dim, store)``; the attention mixer calls
@@ -80,6 +81,16 @@ class StateNeed:
     dtype: torch.dtype = torch.float32
 
 
+@dataclass
+class Term:
+    """One summand of a sublayer's result, for a block that adds the summands to the residual itself (in float32, each
+    with coefficients of its own): ``scale * row[t] * y[t, :]``.  y: [tokens, width] in the activation dtype, or float32
+    planes [planes, tokens, width] that are summed; row: float32 [tokens] (any stride) or None."""
+    y: torch.Tensor
+    scale: float = 1.0
+    row: torch.Tensor = None
+
+
 class Part:
     # True if forward() only launches work on the current stream from device-side data, so that a
     # decode step through this part can be captured into a HIP graph and replayed.  A part that
@@ -128,10 +139,18 @@ class Mixer(Part):
     def forward(self, x, step, view):
         raise NotImplementedError
 
+    def forward_terms(self, x, step, view):
+        """The result as a list of Term whose sum it is; a mixer made of several may hand them on one by one."""
+        return [Term(self.forward(x, step, view))]
+
 
 class FeedForward(Part):
     def forward(self, x, step):
         raise NotImplementedError
+
+    def forward_terms(self, x, step):
+        """The result as a list of Term whose sum it is."""
+        return [Term(self.forward(x, step))]
 
     def forward_after_norm(self, h, delta, norm, step):
         """``forward(norm.add_norm(h, delta), step)``: the pending delta added to the residual stream,

@@ -112,3 +112,65 @@ class ParallelMixerBlock(ParallelBlock):
 
     def _feed_forward(self, xs, step):
         return None
+
+
+class LayerScale(Part):
+    """What a layer with layer scale multiplies its sublayers' results by before they join the residual: a stored
+    vector per sublayer, element by element, and one number for the whole layer (a residual multiplier).
+    params: width, mult (default 1), roles (which sublayers have a vector; default mixer and feed_forward).
+    names: one tensor [width] per role."""
+    graph_safe = True
+
+    def _roles(self):
+        return tuple(self.params.get("roles", ("mixer", "feed_forward")))
+
+    def tensor_specs(self):
+        return {self.names[r]: TensorSpec((self.params["width"],)) for r in self._roles()}
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        self.mult = float(self.params.get("mult", 1.0))
+        self.vectors = {r: tensors[self.names[r]].float().contiguous() for r in self._roles()}
+        self._scaled = {}
+
+    def step_bytes(self, rows):
+        return sum(4 * v.numel() for v in self.vectors.values())
+
+    def coefficient(self, role, factor):
+        """float32 [width]: the role's vector times the layer's multiplier times a summand's own factor."""
+        key = (role, float(factor))
+        if key not in self._scaled:
+            self._scaled[key] = (self.vectors[role].double() * (self.mult * float(factor))).float().contiguous()
+        return self._scaled[key]
+
+    def add(self, h, by_role):
+        """h += sum over roles and their terms of coefficient(role, term.scale) * term.row * term.y, in float32."""
+        terms = [(t.y, self.coefficient(role, t.scale), t.row) for role, ts in by_role for t in ts]
+        limit = self.rt.ops.MAX_ADD_TERMS
+        for at in range(0, len(terms), limit):
+            self.rt.ops.scaled_add(h, terms[at:at + limit])
+        return h
+
+
+class ScaledParallelBlock(Block):
+    """``n = norm(x)``; ``x <- x + mult * (scale_1 * mixer(n) + scale_2 * feed_forward(n))``: one norm, both sublayers
+    read its output, and each result is multiplied element by element by a stored vector before the sum.  The add is
+    one float32 kernel over the sublayers' summands, which arrive apart with their own factors."""
+    roles = {"norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward", "scale": "connection"}
+
+    def _feed_forward(self, x, step):
+        return [("feed_forward", self.feed_forward.forward_terms(x, step))]
+
+    def forward(self, h, delta, step, view):
+        x = self.norm.add_norm(h, delta)
+        terms = [("mixer", self.mixer.forward_terms(x, step, view))] + self._feed_forward(x, step)
+        self.scale.add(h.view(h.shape[0], h.shape[-1]), terms)
+        return None
+
+
+class ScaledParallelMixerBlock(ScaledParallelBlock):
+    """The same without a feed-forward."""
+    roles = {"norm": "norm", "mixer": "mixer", "scale": "connection"}
+
+    def _feed_forward(self, x, step):
+        return []

@@ -8,41 +8,61 @@ or value.  The heads' weights are then mixed, ``w'_h = sum_g talk[h, g] w_g``, a
 weights to the values of its own key-value head.  Keys and values may differ in head size.  A layer that
 borrows (``borrows=True``) has no key and value projections and reads the keys (as cached, rotated) and values
 that an earlier layer keeps, with queries, window, sink and mixing of its own.  Scores, softmax and the mixing
-are float32 in every mode."""
+are float32 in every mode.
+
+Variants by parameter: no biases at all (``bias=False``); turning pairs of adjacent lanes ``(2i, 2i + 1)``
+(``pairing="adjacent"``); values that are the keys as projected, before the rotation, with no value projection
+(``values="keys"``; then ``vdim = dim``)."""
 from __future__ import annotations
 
 import os
 
 import torch
 
-from .base import KVNeed, Mixer, TensorSpec
+from .base import KVNeed, Mixer, TensorSpec, Term
 
 
 class SinkAttention(Mixer):
     """params: width, heads, kv_heads, dim, vdim, scale, window (0: all keys), cache_window (what the cache keeps:
     the largest window of this layer and of the layers that borrow from it; default window), rot_dims, position
     (a rotary encoding whose table has rot_dims/2 pairs; given by the model builder), borrows, sink, talk (whether
-    the layer has them; default True).
-    names: q, q_bias, o, o_bias, sink, talk and, unless the layer borrows, k, k_bias, v, v_bias."""
+    the layer has them; default True), bias (whether the projections have biases; default True), pairing ("half",
+    the default: lane i turns with lane i + rot_dims/2; "adjacent": lane 2i with 2i + 1), values ("projected", the
+    default, or "keys": the unrotated keys are the values and there is no value projection).
+    names: q, q_bias, o, o_bias, sink, talk and, unless the layer borrows, k, k_bias, v, v_bias (those the parameters
+    leave)."""
     graph_safe = True
 
     def _flags(self):
         p = self.params
         return bool(p.get("borrows")), p.get("sink", True), p.get("talk", True)
 
+    def _variant(self):
+        """(projections have biases, values are the keys, pairs are adjacent lanes)"""
+        p = self.params
+        values, pairing = p.get("values", "projected"), p.get("pairing", "half")
+        if values not in ("projected", "keys") or pairing not in ("half", "adjacent"):
+            raise ValueError(f"sink attention: values={values!r} (projected, keys) or pairing={pairing!r} (half, adjacent) unknown")
+        if values == "keys" and (p["vdim"] != p["dim"] or p.get("borrows")):
+            raise ValueError("values that are the keys have the keys' head size, and their layer keeps its own")
+        return bool(p.get("bias", True)), values == "keys", pairing == "adjacent"
+
     def tensor_specs(self):
         p, n = self.params, self.names
         d, H, G, dk, dv = p["width"], p["heads"], p["kv_heads"], p["dim"], p["vdim"]
         borrows, sink, talk = self._flags()
-        specs = {n["q"]: TensorSpec((H * dk, d)), n["q_bias"]: TensorSpec((H * dk,)),
-                 n["o"]: TensorSpec((d, H * dv)), n["o_bias"]: TensorSpec((d,))}
+        bias, values_are_keys, _ = self._variant()
+        specs = {n["q"]: TensorSpec((H * dk, d)), n["o"]: TensorSpec((d, H * dv))}
         if sink:
             specs[n["sink"]] = TensorSpec((H,))
         if talk:
             specs[n["talk"]] = TensorSpec((H, H))
         if not borrows:
-            specs.update({n["k"]: TensorSpec((G * dk, d)), n["k_bias"]: TensorSpec((G * dk,)),
-                          n["v"]: TensorSpec((G * dv, d)), n["v_bias"]: TensorSpec((G * dv,))})
+            specs[n["k"]] = TensorSpec((G * dk, d))
+            if not values_are_keys:
+                specs[n["v"]] = TensorSpec((G * dv, d))
+        if bias:
+            specs.update({n[r + "_bias"]: TensorSpec(specs[n[r]].shape[:1]) for r in ("q", "o", "k", "v") if n.get(r) in specs})
         return specs
 
     def cache_need(self):
@@ -57,10 +77,11 @@ class SinkAttention(Mixer):
             raise ValueError(f"{self.H} heads are no multiple of {self.G} key-value heads")
         self.scale, self.window, self.rot = float(p["scale"]), int(p.get("window", 0)), int(p.get("rot_dims", 0))
         self.borrows, sink, talk = self._flags()
+        bias, self.values_are_keys, self.adjacent = self._variant()
         self.position = p.get("position")
         if self.rot and (self.position is None or self.rot % 2 or self.rot > self.dk):
             raise ValueError("rot_dims must be even, at most the key head size, and come with a rotary encoding")
-        roles = ("q",) if self.borrows else ("q", "k", "v")
+        roles = ("q",) if self.borrows else ("q", "k") if self.values_are_keys else ("q", "k", "v")
         ws = [tensors[n[r]] for r in roles]
         if len({w.dtype for w in ws}) != 1:
             ws = [w.float() for w in ws]
@@ -68,9 +89,9 @@ class SinkAttention(Mixer):
         if rows % 8:
             ws.append(torch.zeros(8 - rows % 8, ws[0].shape[1], dtype=ws[0].dtype, device=ws[0].device))
         self.w_in = rt.weight(torch.cat(ws, dim=0))
-        self.bias_in = torch.cat([tensors[n[r + "_bias"]].float() for r in roles]).contiguous()
+        self.bias_in = torch.cat([tensors[n[r + "_bias"]].float() for r in roles]).contiguous() if bias else None
         self.w_o = rt.weight(tensors[n["o"]])
-        self.output_bias = tensors[n["o_bias"]].float().contiguous()
+        self.output_bias = tensors[n["o_bias"]].float().contiguous() if bias else None
         self.on_matrix_cores = rt.ops.sink_attn_mfma_supported(rt.dtype, self.dk, self.dv) and self.scale > 0 \
             and os.environ.get("BURN_LM_AMD_SINK_ATTENTION") != "generic"
         if self.on_matrix_cores:
@@ -94,12 +115,17 @@ class SinkAttention(Mixer):
     def forward(self, x, step, view):
         """The whole mixer, its output bias added."""
         out = self.rt.linear(self.attend(self.project(x, step, view), step, view), self.w_o)
-        return out.add_(self.output_bias.to(out.dtype))
+        return out.add_(self.output_bias.to(out.dtype)) if self.output_bias is not None else out
 
     def forward_unbiased(self, x, step, view):
         """(result without the output projection's bias, possibly as partial planes; that bias in float32): for a
         block that adds both to the residual stream itself."""
         return self.output(self.attend(self.project(x, step, view), step, view)), self.output_bias
+
+    def forward_terms(self, x, step, view):
+        if self.output_bias is not None:
+            return super().forward_terms(x, step, view)
+        return [Term(self.forward_unbiased(x, step, view)[0])]
 
     def project(self, x, step, view):
         """q (and k, v) of the step's tokens with their biases, q and k turned by position, k and v stored."""
@@ -114,7 +140,7 @@ class SinkAttention(Mixer):
             raise ValueError("a layer with key and value projections keeps its own pages, a borrowing layer reads another's")
         rt.ops.qkv_prepare(qkv, self.bias_in, self.position.table if self.rot else None, self.rot, step,
                            view.block_table(step), view.k, view.v, view.page_size, self.H, self.G, self.dk, self.dv,
-                           write_kv=store)
+                           write_kv=store, adjacent=self.adjacent, values_are_keys=self.values_are_keys)
         return qkv
 
     def attend(self, qkv, step, view):
