@@ -342,7 +342,22 @@ def digasun_config(width, ff, heads, layers, vocab):
                 norm=dict(eps=1e-6), token_side=dict(dim=64), layers=made)
 
 
-DESIGNS = {"fuvirax": fuvirax_config, "digasun": digasun_config}
+def girelix_config(width, ff, heads, layers, vocab):
+    """Every layer: softmax attention over all earlier keys (heads of 128 lanes in groups of four, values that are the
+    keys, a sink) beside lightning attention (as many heads of 128 x 128), and 16 experts of 512 (as many weights as the
+    Llama's feed-forward) with 4 pass-through experts, 4 chosen within 2 of 4 groups."""
+    moe = dict(kind="moe", expert=dict(ff=512), router=dict(experts=16, identity=4, top=4, groups=dict(count=4, keep=2)))
+    mixer = dict(left=dict(heads=heads, kv_heads=heads // 4, dim=128, vdim=128, scale=128 ** -0.5,
+                           rot=dict(base=500000.0, dims=128)),
+                 right=dict(heads=heads, dim=128, vdim=128, decay=[1.0 - 2.0 ** -(2 + 6 * h / heads) for h in range(heads)]),
+                 left_scale=0.8, right_scale=1.1)
+    return dict(architecture="Girelix", vocab=vocab, width=width, norm=dict(eps=1e-6), residual_mult=0.7,
+                layers=[dict(type="parallel", mixer=mixer, mlp=moe) for _ in range(layers)])
+
+
+DESIGNS = {"fuvirax": fuvirax_config, "digasun": digasun_config, "girelix": girelix_config}
+# the designs that run beside one (the Llama of equal size always does): the closest of those that were there before
+BESIDE = {"girelix": ("digasun",)}
 
 
 def mixer_rates(engine, batch, context, prefill_tokens):
@@ -352,20 +367,21 @@ def mixer_rates(engine, batch, context, prefill_tokens):
     import torch
     rt, model = engine.rt, engine.model
     out, seen = {}, {}
-    for i, pl in enumerate(model.plan.order):
-        m = model.blocks[pl.layer].mixer
-        if getattr(m, "borrows", False):
-            continue
-        seen.setdefault(type(m).__name__, (model.blocks[pl.layer], engine.cache.views[i]))
-    width = model.plan.width
-
     def mixer_view(block, view):
         if hasattr(block, "_mixer_view"):
             return block._mixer_view(view)
         return block._views(view)[1] if hasattr(block, "_views") else view
 
-    def run(kind, block, view, step, x, tag, nbytes=None, flops=None):
-        m, v = block.mixer, mixer_view(block, view)
+    for i, pl in enumerate(model.plan.order):
+        block = model.blocks[pl.layer]
+        m, v = block.mixer, mixer_view(block, engine.cache.views[i])
+        # a pair of mixers side by side: each of the two with its own view
+        for one, view in (zip(m.sides, m._views(v)) if hasattr(m, "sides") else ((m, v),)):
+            if not getattr(one, "borrows", False):
+                seen.setdefault(type(one).__name__, (one, view))
+    width = model.plan.width
+
+    def run(kind, m, v, step, x, tag, nbytes=None, flops=None):
         if kind == "Attention":
             mid, mix = m.project(x, step, v), m.attend
         elif kind == "LatentAttention":
@@ -379,6 +395,8 @@ def mixer_rates(engine, batch, context, prefill_tokens):
                 return
             mid, mix = m.project(x, step, v), m.attend
         elif kind == "GatedLinearAttention":
+            mid, mix = m.project(x), m.scan
+        elif kind == "LightningAttention":
             mid, mix = m.project(x), m.scan
         else:
             return
@@ -415,8 +433,8 @@ def mixer_rates(engine, batch, context, prefill_tokens):
         engine.cache.advance(s, context - 1)
     step = engine.build_step([(s, [1], [0]) for s in slots])
     x = torch.randn(batch, width, device=rt.device).to(rt.dtype)
-    for kind, (block, view) in seen.items():
-        run(kind, block, view, step, x, "decode", nbytes=state_bytes(view))
+    for kind, (mixer, view) in seen.items():
+        run(kind, mixer, view, step, x, "decode", nbytes=state_bytes(view))
     for s in slots:
         engine.close(s)
     T = prefill_tokens
@@ -424,15 +442,16 @@ def mixer_rates(engine, batch, context, prefill_tokens):
     engine.cache.reserve([(s, T)])
     step = engine.build_step([(s, [1] * T, [T - 1])])
     x = torch.randn(T, width, device=rt.device).to(rt.dtype)
-    for kind, (block, view) in seen.items():
-        run(kind, block, view, step, x, "prefill", flops=block.mixer.mixing_flops(0, T))
+    for kind, (mixer, view) in seen.items():
+        run(kind, mixer, view, step, x, "prefill", flops=mixer.mixing_flops(0, T))
     engine.close(s)
     return out
 
 
 def run_design(args):
-    """--design fuvirax | digasun: prompt and decode throughput of the design at sizes that resemble a real model's layers
-    (random weights), beside the Llama of equal size, and the mixing kernels of both alone against their limits."""
+    """--design fuvirax | digasun | girelix: prompt and decode throughput of the design at sizes that resemble a real
+    model's layers (random weights), beside the Llama of equal size (and, for a design that has one, the closest earlier
+    design), and the mixing kernels of all alone against their limits."""
     import torch
     from burn_lm_amd.config.presets import preset
     from burn_lm_amd.engine.loading import random_engine
@@ -448,8 +467,9 @@ def run_design(args):
         size = DESIGN_SIZES[name]
         base = preset(size["llama"])
         base["num_hidden_layers"] = layers
-        configs = {args.design: DESIGNS[args.design](size["width"], size["ff"], size["heads"], layers, base["vocab_size"]),
-                   "llama": base}
+        configs = {d: DESIGNS[d](size["width"], size["ff"], size["heads"], layers, base["vocab_size"])
+                   for d in (args.design,) + BESIDE.get(args.design, ())}
+        configs["llama"] = base
         entry = {}
         for model, config in configs.items():
             print(f"[bench] {name} {model}: building", file=sys.stderr, flush=True)
@@ -532,7 +552,7 @@ def main():
                          "launched kernel by kernel on a cache that is filled without a prompt step; prints its time and "
                          "no JSON line, and says on stderr where it is")
     ap.add_argument("--design", default=None, metavar="NAME",
-                    help="instead of the default measurement: prompt and decode throughput of a design (fuvirax, digasun) at model-like "
+                    help="instead of the default measurement: prompt and decode throughput of a design (fuvirax, digasun, girelix) at model-like "
                          "layer sizes beside the Llama of equal size, with the mixing kernels alone (--layers, default 6; "
                          "--sizes 1b-like,3b-like)")
     ap.add_argument("--sizes", default=None, help="with --design: which of its sizes, with commas between them")
@@ -555,9 +575,14 @@ def main():
             print(f"[bench] {what}", file=sys.stderr, flush=True)
 
     config = preset(args.preset)
-    full_layers = config["num_hidden_layers"]
-    layers = args.layers or full_layers
-    config["num_hidden_layers"] = layers
+    if isinstance(config.get("layers"), list):      # a design whose config.json lists its layers (only with --profile)
+        full_layers = len(config["layers"])
+        layers = args.layers or full_layers
+        config["layers"] = config["layers"][:layers]
+    else:
+        full_layers = config["num_hidden_layers"]
+        layers = args.layers or full_layers
+        config["num_hidden_layers"] = layers
     biggest = max(args.batch, 1 if args.no_points else 64)
     from burn_lm_amd.csrc import build as _build
     if args.profile:

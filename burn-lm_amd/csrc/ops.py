@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 33
+ABI_VERSION = 34
 _lib = None
 _lock = threading.Lock()
 
@@ -1258,7 +1258,8 @@ def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, st
     updated; o_raw: zeroed float32 [T, H * dv]; out [T, H * dv] in proj's dtype.  segments: (count, tokens each) as
     gla_segments gives them (the default), or (1, 0) for one walk per sequence.
     The same recurrence with other surroundings: fixed_decay (float32 [H * dk]): the decays of every token, in place of
-    decay_in, decay_bias and tau (which are then None); activation "silu": on queries, keys and values; q_scale: the
+    decay_in, decay_bias and tau (which are then None); activation "silu": on queries, keys and values, rounded to
+    proj's dtype (where the sequences are walked in segments, proj's first columns are activated in place); q_scale: the
     queries' factor (default dk^-1/2); norm_all: one root mean square over all heads' lanes, norm_w [H * dv] (default:
     per head, norm_w [dv]); gate: "silu" or "sigmoid" of the output gate's logits."""
     _gpu(proj, decay_in, decay_bias, norm_w, state, o_raw, out, fixed_decay)

@@ -518,61 +518,121 @@ extern "C" int blm_scaled_add(float* h, int T, int D, int n_terms,
 // chosen pass-through experts.
 // ---------------------------------------------------------------------------------------
 #define PB_MAX_ROUTED 256
-__global__ void moe_route_grouped_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction,
-                                         int E, int n_identity, int groups, int keep, int top, float* __restrict__ weights,
-                                         int T) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+#define PB_ROUTED_PER_LANE (PB_MAX_ROUTED / BLM_WAVE)
+
+// the largest (value, index) pair over a wavefront; of equal values the one with the lower index
+__device__ __forceinline__ void pb_wave_best(float& v, int& i) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(v, off);
+    const int oi = __shfl_xor(i, off);
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+  }
+}
+
+// One wavefront per token; lane l holds the experts l, l + 64, ...  Scores and corrected scores stay in registers; the
+// groups' ranks and the kept groups pass through the wavefront's piece of shared memory.
+__global__ void __launch_bounds__(256)
+    moe_route_grouped_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction, int E,
+                             int n_identity, int groups, int keep, int top, float* __restrict__ weights, int T) {
+  __shared__ float sm_choice[4][PB_MAX_ROUTED];
+  __shared__ int sm_kept[4][PB_MAX_ROUTED];
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;
   const int N = E + n_identity;
   const float* z = logits + (size_t)t * ld;
   float* w = weights + (size_t)t * (E + 1);
-  float largest = z[0];
-  for (int e = 1; e < N; ++e) largest = fmaxf(largest, z[e]);
+  float zs[PB_ROUTED_PER_LANE], score[PB_ROUTED_PER_LANE], choice[PB_ROUTED_PER_LANE];
+  float largest = -INFINITY;
+#pragma unroll
+  for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) {
+    const int e = lane + k * BLM_WAVE;
+    zs[k] = e < N ? z[e] : -INFINITY;
+    largest = fmaxf(largest, zs[k]);
+  }
+  largest = wave_max(largest);
   float denom = 0.f;
-  for (int e = 0; e < N; ++e) denom += expf(z[e] - largest);
-  const float inv = 1.0f / denom;
-  auto score = [&](int e) { return expf(z[e] - largest) * inv; };
-  auto choice = [&](int e) { return score(e) + (correction ? correction[e] : 0.f); };
-  // the groups that stay: `keep` times the best group not yet taken (a bit per group)
-  unsigned long long kept[PB_MAX_ROUTED / 64] = {0ull, 0ull, 0ull, 0ull};
-  const int per = groups > 1 ? N / groups : N;
+#pragma unroll
+  for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) {
+    score[k] = lane + k * BLM_WAVE < N ? expf(zs[k] - largest) : 0.f;
+    denom += score[k];
+  }
+  const float inv = 1.0f / wave_sum(denom);
+#pragma unroll
+  for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) {
+    const int e = lane + k * BLM_WAVE;
+    score[k] *= inv;
+    choice[k] = e < N ? score[k] + (correction ? correction[e] : 0.f) : -INFINITY;
+  }
   if (groups > 1) {
-    for (int k = 0; k < keep; ++k) {
-      int best = -1;
+    const int per = N / groups;
+#pragma unroll
+    for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) {
+      const int e = lane + k * BLM_WAVE;
+      if (e < N) { sm_choice[wave][e] = choice[k]; sm_kept[wave][e] = 0; }
+    }
+    __builtin_amdgcn_wave_barrier();
+    float rank[PB_ROUTED_PER_LANE];      // of group lane + k * 64: its largest corrected score
+#pragma unroll
+    for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) {
+      const int g = lane + k * BLM_WAVE;
+      rank[k] = -INFINITY;
+      if (g < groups)
+        for (int e = g * per; e < (g + 1) * per; ++e) rank[k] = fmaxf(rank[k], sm_choice[wave][e]);
+    }
+    bool running[PB_ROUTED_PER_LANE];
+#pragma unroll
+    for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) running[k] = lane + k * BLM_WAVE < groups;
+    for (int n = 0; n < keep; ++n) {
       float bv = -INFINITY;
-      for (int g = 0; g < groups; ++g) {
-        if (kept[g >> 6] >> (g & 63) & 1ull) continue;
-        float gv = -INFINITY;
-        for (int e = g * per; e < (g + 1) * per; ++e) gv = fmaxf(gv, choice(e));
-        if (best < 0 || gv > bv) { best = g; bv = gv; }
-      }
-      kept[best >> 6] |= 1ull << (best & 63);
+      int bi = 0x7fffffff;      // no group
+#pragma unroll
+      for (int k = 0; k < PB_ROUTED_PER_LANE; ++k)
+        if (running[k] && (bi == 0x7fffffff || rank[k] > bv)) { bv = rank[k]; bi = lane + k * BLM_WAVE; }
+      pb_wave_best(bv, bi);
+#pragma unroll
+      for (int k = 0; k < PB_ROUTED_PER_LANE; ++k)
+        if (lane + k * BLM_WAVE == bi) { running[k] = false; sm_kept[wave][bi] = 1; }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) {
+      const int e = lane + k * BLM_WAVE;
+      if (e < N && !sm_kept[wave][e / per]) choice[k] = -INFINITY;
     }
   }
-  for (int e = 0; e <= E; ++e) w[e] = 0.f;
-  int chosen[PB_MAX_TOP];
-  float val[PB_MAX_TOP];
+  // the `top` largest corrected scores, one after the other; a chosen expert leaves the running
+  bool mine[PB_ROUTED_PER_LANE], open[PB_ROUTED_PER_LANE];
+#pragma unroll
+  for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) {
+    mine[k] = false;
+    open[k] = lane + k * BLM_WAVE < N && choice[k] != -INFINITY;      // experts of groups left out never run
+  }
   float sum = 0.f;
-  for (int k = 0; k < top; ++k) {
-    int best = -1;
+  for (int n = 0; n < top; ++n) {
     float bv = -INFINITY;
-    for (int e = 0; e < N; ++e) {
-      if (groups > 1) {
-        const int g = e / per;
-        if (!(kept[g >> 6] >> (g & 63) & 1ull)) continue;
-      }
-      bool taken = false;
-      for (int j = 0; j < k; ++j) taken |= chosen[j] == e;
-      if (taken) continue;
-      const float v = choice(e);
-      if (best < 0 || v > bv) { best = e; bv = v; }
-    }
-    chosen[k] = best;
-    val[k] = score(best);
-    sum += val[k];
+    int bi = 0x7fffffff;      // no expert
+#pragma unroll
+    for (int k = 0; k < PB_ROUTED_PER_LANE; ++k)
+      if (open[k] && (bi == 0x7fffffff || choice[k] > bv)) { bv = choice[k]; bi = lane + k * BLM_WAVE; }
+    pb_wave_best(bv, bi);
+#pragma unroll
+    for (int k = 0; k < PB_ROUTED_PER_LANE; ++k)
+      if (lane + k * BLM_WAVE == bi) { mine[k] = true; open[k] = false; sum += score[k]; }
   }
+  sum = wave_sum(sum);
   const float norm = 1.0f / (sum + 1e-20f);
-  for (int k = 0; k < top; ++k) w[chosen[k] < E ? chosen[k] : E] += val[k] * norm;
+  // real experts' weights straight out; the pass-through experts' added up over the wavefront
+  float passed = 0.f;
+#pragma unroll
+  for (int k = 0; k < PB_ROUTED_PER_LANE; ++k) {
+    const int e = lane + k * BLM_WAVE;
+    if (e < E) w[e] = mine[k] ? score[k] * norm : 0.f;
+    else if (e < N && mine[k]) passed += score[k] * norm;
+  }
+  passed = wave_sum(passed);
+  if (lane == 0) w[E] = passed;
 }
 
 extern "C" int blm_moe_route_grouped(const float* logits, int ld, const float* correction, int E, int n_identity, int groups,
@@ -584,7 +644,7 @@ extern "C" int blm_moe_route_grouped(const float* logits, int ld, const float* c
   BLM_REQUIRE(groups <= 1 || (N % groups == 0 && keep >= 1 && keep <= groups), "moe_route_grouped: %d experts in %d groups, %d kept",
               N, groups, keep);
   BLM_REQUIRE(top <= (groups > 1 ? keep * (N / groups) : N), "moe_route_grouped: top=%d is more than the kept groups hold", top);
-  hipLaunchKernelGGL(moe_route_grouped_kernel, dim3((T + 127) / 128), dim3(128), 0, stream, logits, ld, correction, E,
+  hipLaunchKernelGGL(moe_route_grouped_kernel, dim3((T + 3) / 4), dim3(256), 0, stream, logits, ld, correction, E,
                      n_identity, groups, keep, top, weights, T);
   BLM_LAUNCH_CHECK("moe_route_grouped");
   return 0;

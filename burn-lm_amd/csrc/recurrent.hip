@@ -197,8 +197,58 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
   }
 }
 
+// The same for rows of many lanes (a norm over all heads' lanes together): a block of four wavefronts per row, the
+// row's values kept in registers between the two passes (up to HEAD_NORM_WIDE_PER per thread, else read again).
+#define HEAD_NORM_WIDE_PER 8
+template <typename TA>
+__global__ void __launch_bounds__(256)
+    head_norm_wide_kernel(const float* __restrict__ o_raw, const float* __restrict__ norm_w, const TA* __restrict__ gate,
+                          int gate_ld, int gate_mode, int H, TA* __restrict__ out, int dv, float eps) {
+  __shared__ float part[4];
+  const long long item = blockIdx.x;
+  const float* src = o_raw + (size_t)item * dv;
+  const TA* grow = gate ? gate + (size_t)(item / H) * gate_ld + (size_t)(item % H) * dv : nullptr;
+  float x[HEAD_NORM_WIDE_PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < HEAD_NORM_WIDE_PER; ++k) {
+    const int j = threadIdx.x + k * 256;
+    x[k] = j < dv ? src[j] : 0.f;
+    ss = fmaf(x[k], x[k], ss);
+  }
+  for (int j = threadIdx.x + HEAD_NORM_WIDE_PER * 256; j < dv; j += 256) ss = fmaf(src[j], src[j], ss);
+  ss = wave_sum(ss);
+  if ((threadIdx.x & (BLM_WAVE - 1)) == 0) part[threadIdx.x / BLM_WAVE] = ss;
+  __syncthreads();
+  const float inv = 1.0f / sqrtf((part[0] + part[1] + part[2] + part[3]) / (float)dv + eps);
+  auto put = [&](int j, float xv) {
+    float v = xv * inv * norm_w[j];
+    if (grow) {
+      const float z = to_float(grow[j]);
+      v *= gate_mode == 2 ? blm_silu(z) : blm_sigmoid(z);
+    }
+    out[(size_t)item * dv + j] = from_float<TA>(v);
+  };
+#pragma unroll
+  for (int k = 0; k < HEAD_NORM_WIDE_PER; ++k) {
+    const int j = threadIdx.x + k * 256;
+    if (j < dv) put(j, x[k]);
+  }
+  for (int j = threadIdx.x + HEAD_NORM_WIDE_PER * 256; j < dv; j += 256) put(j, src[j]);
+}
+
 static int launch_head_norm(const float* o_raw, const float* norm_w, const void* gate, int gate_ld, int gate_mode, int H,
                             void* out, int dtype, long long items, int dv, float eps, hipStream_t stream) {
+  if (dv >= 512 && items < (1ll << 31)) {
+    if (dtype == BLM_F32)
+      hipLaunchKernelGGL(head_norm_wide_kernel<float>, dim3((unsigned)items), dim3(256), 0, stream, o_raw, norm_w,
+                         (const float*)gate, gate_ld, gate_mode, H, (float*)out, dv, eps);
+    else
+      hipLaunchKernelGGL(head_norm_wide_kernel<bf16>, dim3((unsigned)items), dim3(256), 0, stream, o_raw, norm_w,
+                         (const bf16*)gate, gate_ld, gate_mode, H, (bf16*)out, dv, eps);
+    BLM_LAUNCH_CHECK("head_norm_wide");
+    return 0;
+  }
   const unsigned blocks = (unsigned)((items + SCAN_WAVES - 1) / SCAN_WAVES);
   if (dtype == BLM_F32)
     hipLaunchKernelGGL(head_norm_kernel<float>, dim3(blocks), dim3(SCAN_WAVES * BLM_WAVE), 0, stream, o_raw, norm_w,
@@ -575,6 +625,19 @@ __global__ void gla_gates_kernel(const TA* __restrict__ decay_in, const float* _
     gates[e] = expf(-blm_softplus(-(to_float(decay_in[e]) + bias[e % HK])) * inv_tau);
 }
 
+// SiLU in place on the first `cols` columns of every row (queries, keys and values of a step whose sequences are walked
+// in segments: there every column group of a head would otherwise activate the head's queries and keys again).  The
+// result is rounded to the rows' type, as the walk that activates on the way rounds it.
+template <typename TA>
+__global__ void silu_rows_kernel(TA* __restrict__ proj, int ld, int cols, long long n) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const long long t = e / cols;
+    TA* at = proj + (size_t)t * ld + (e - t * cols);
+    *at = from_float<TA>(blm_silu(to_float(*at)));
+  }
+}
+
 // With SEG a sequence's tokens are cut into n_seg segments of seg_len tokens that different wavefronts walk at the
 // same time: the first from the sequence's state, the others from zero.  The recurrence is linear in the state, so
 //   S_t = (prod of the segment's decays up to t) S_start + (what the walk from zero gives),
@@ -634,12 +697,12 @@ __global__ void __launch_bounds__(SCAN_WAVES* BLM_WAVE)
           if (i < dk) {
             raw_d[tt][k] = gr[h * dk + i];
             const float kx = to_float(row[(size_t)H * dk + h * dk + i]), qx = to_float(row[h * dk + i]);
-            raw_k[tt][k] = act ? blm_silu(kx) : kx;
-            raw_q[tt][k] = (act ? blm_silu(qx) : qx) * q_scale;
+            raw_k[tt][k] = act ? to_float(from_float<TA>(blm_silu(kx))) : kx;
+            raw_q[tt][k] = (act ? to_float(from_float<TA>(blm_silu(qx))) : qx) * q_scale;
           }
         }
         v_in[tt] = own ? to_float(row[(size_t)2 * H * dk + h * dv + col]) : 0.f;
-        if (act) v_in[tt] = blm_silu(v_in[tt]);
+        if (act) v_in[tt] = to_float(from_float<TA>(blm_silu(v_in[tt])));
       }
     }
   };
@@ -789,10 +852,11 @@ __global__ void __launch_bounds__(BLM_WAVE)
 // Variants of the same recurrence, for mixers that differ in what surrounds it:
 //   fixed_decay [H*dk] float (not null): every token's decays, instead of decay_in, decay_bias and tau (a decay per head that
 //     is a constant of the model; gates is then not used);
-//   act_mode 1: SiLU on the queries, keys and values as they are read;  q_scale: the queries' factor (<= 0: dk^-1/2);
+//   act_mode 1: SiLU on the queries, keys and values (rounded to the rows' type) as they are read, or, where the sequences
+//     are walked in segments, in place beforehand: proj is then changed;  q_scale: the queries' factor (<= 0: dk^-1/2);
 //   norm_all 1: the root mean square is taken over all heads' value lanes together and norm_w is [H*dv];
 //   gate_mode: 1 sigmoid, 2 SiLU of the output gate's logits.
-extern "C" int blm_gla_scan(const void* proj, int dtype, int ld, const void* decay_in, const float* decay_bias, float tau,
+extern "C" int blm_gla_scan(void* proj, int dtype, int ld, const void* decay_in, const float* decay_bias, float tau,
                             const float* norm_w, float eps, float* state, float* gates, float* o_raw, void* out,
                             const int* cu_seqlens, const int* seq_slots, int T, int B, int H, int dk, int dv, int max_new,
                             int n_seg, int seg_len, float* seg_end, float* seg_start, float* seg_decay, float* q_tilde,
@@ -815,6 +879,15 @@ extern "C" int blm_gla_scan(const void* proj, int dtype, int ld, const void* dec
     else
       hipLaunchKernelGGL(gla_gates_kernel<bf16>, dim3(gblocks), dim3(256), 0, stream, (const bf16*)decay_in, decay_bias, 1.0f / tau, gates, n, H * dk);
     BLM_LAUNCH_CHECK("gla_gates");
+  }
+  if (act_mode == 1 && n_seg > 1) {
+    const int cols = 2 * H * dk + H * dv;
+    const long long n = (long long)T * cols;
+    const unsigned ablocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+    if (dtype == BLM_F32) hipLaunchKernelGGL(silu_rows_kernel<float>, dim3(ablocks), dim3(256), 0, stream, (float*)proj, ld, cols, n);
+    else hipLaunchKernelGGL(silu_rows_kernel<bf16>, dim3(ablocks), dim3(256), 0, stream, (bf16*)proj, ld, cols, n);
+    BLM_LAUNCH_CHECK("silu_rows");
+    act_mode = 0;
   }
   const float q_scale = q_scale_in > 0.f ? q_scale_in : 1.0f / sqrtf((float)dk);
   const float* decays = fixed_decay ? fixed_decay : gates;

@@ -514,17 +514,18 @@ def test_keys_are_turned_in_adjacent_pairs_and_kept_unturned_as_values(dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
-def test_fading_state_kernel_against_the_plain_function(dtype):
+@pytest.mark.parametrize("H,dk,dv", [(3, 12, 20), (10, 4, 250)], ids=["small", "norm_over_2500_lanes"])
+def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv):
     """Three sequences in one step: a long prompt (walked in segments), a continuation from a state, one token from a
     state; heads that forget at once, slowly and never; a state slot that is not in the step stays as it was.  The
     recurrence is written out here once more, on rows that stand for the projections' results."""
     from burn_lm_amd.csrc import ops
     dev = "cuda"
-    H, dk, dv, D = 3, 12, 20, 16
-    r = dict(heads=H, dim=dk, vdim=dv, decay=[0.05, 0.999, 1.0])
+    r = dict(heads=H, dim=dk, vdim=dv, decay=([0.05, 0.999, 1.0] * 4)[:H])
     rng = np.random.default_rng(4)
     bf = lambda a: torch.from_numpy(np.asarray(a, dtype=np.float32)).to(dtype).double().numpy()
     W = {"r.norm": rng.uniform(0.5, 1.5, H * dv)}
+    act = lambda z: bf(P.silu(z))            # the activations are rounded to the rows' type
     news, slots = [300, 40, 1], [2, 0, 3]
     states = rng.standard_normal((4, H, dk, dv))
     states[2] = 0.0
@@ -539,8 +540,8 @@ def test_fading_state_kernel_against_the_plain_function(dtype):
         o = np.zeros((n, H, dv))
         for t in range(n):
             for hd in range(H):
-                S[hd] = r["decay"][hd] * S[hd] + np.outer(P.silu(k[t].reshape(H, dk)[hd]), P.silu(v[t].reshape(H, dv)[hd]))
-                o[t, hd] = S[hd].T @ P.silu(q[t].reshape(H, dk)[hd])
+                S[hd] = r["decay"][hd] * S[hd] + np.outer(act(k[t].reshape(H, dk)[hd]), act(v[t].reshape(H, dv)[hd]))
+                o[t, hd] = S[hd].T @ act(q[t].reshape(H, dk)[hd])
         want.append((P.rms_norm(o.reshape(n, H * dv), W["r.norm"], 1e-5) * P.sigmoid(gl), S))
         at += n
     step = _Step(news, [0, 77, 500], slots, dev)
