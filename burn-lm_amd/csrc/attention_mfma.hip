@@ -307,7 +307,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
                              const int* __restrict__ positions, const int* __restrict__ cu_seqlens,
                              const int* __restrict__ block_table, int table_width,
                              const bf16* __restrict__ kcache, const bf16* __restrict__ vcache, int nh, int nkv,
-                             float scale, int window) {
+                             float scale, int window, const float* __restrict__ sinks) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
   // Head sizes 64 and 128: a page comes straight from global memory into shared memory, its rows'
@@ -365,8 +365,10 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 
   uint4 qf[KS];
   load_q<HD>(q + (size_t)row * q_row_stride + (size_t)head * HD, qf);
-  float m = -INFINITY;
-  f32x4_t lsum = {0.f, 0.f, 0.f, 0.f};   // the denominator of query column c, the same in all four places
+  // a sink (one logit per head, not scaled, no value) is a share of the denominator from the start
+  float m = sinks ? sinks[head] * 1.4426950408889634f : -INFINITY;
+  const float l0 = sinks ? 1.f : 0.f;
+  f32x4_t lsum = {l0, l0, l0, l0};   // the denominator of query column c, the same in all four places
   f32x4_t o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -601,7 +603,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
                           const int* __restrict__ positions, const int* __restrict__ cu_seqlens,
                           const int* __restrict__ block_table, int table_width,
                           const bf16* __restrict__ kcache, const bf16* __restrict__ vcache, int nh, int nkv,
-                          float scale, int window) {
+                          float scale, int window, const float* __restrict__ sinks) {
   static_assert(HD % 32 == 0 && HD <= 128, "32-query prefill: head sizes 32, 64, 96, 128");
   constexpr int KS = HD / 16, RT = HD / 32, QT = 32;
   constexpr bool DIRECT = HD == 64 || HD == 128;   // as in the 16-query kernel
@@ -653,8 +655,8 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE) __attribute__((amdgpu_wave
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 16 + hb * 8);
   }
-  float m = -INFINITY;
-  float lsum = 0.f;
+  float m = sinks ? sinks[head] * 1.4426950408889634f : -INFINITY;     // a sink: see the 16-query kernel
+  float lsum = (sinks && hb == 0) ? 1.f : 0.f;                          // the two lanes of a query add theirs up
   f32x16_t o[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
@@ -757,7 +759,7 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
                             const int* __restrict__ token_seq, const int* __restrict__ block_table,
                             int table_width, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
                             int nh, int nkv, float scale, int window, int n_splits, float* part_o,
-                            float* part_ml, int* arrivals, bf16* out) {
+                            float* part_ml, int* arrivals, bf16* out, const float* __restrict__ sinks) {
   constexpr int KS = (HD + 31) / 32;
   constexpr int DT = (HD + 15) / 16;
   // Every wavefront brings its pages through a staging area of its own in shared memory: whole
@@ -787,8 +789,11 @@ __global__ void __launch_bounds__(AM_WAVES* BLM_WAVE)
   const int b = token_seq[t];
   const int head = kvh * G + min(g0 + c, G - 1);   // columns past the group's end repeat its last head
 
-  float m = -INFINITY;
-  f32x4_t lsum = {0.f, 0.f, 0.f, 0.f};   // the denominator of query column c, the same in all four places
+  // a sink counts once per (token, head): with the first wavefront of the first split
+  const bool has_sink = sinks != nullptr && split == 0 && wave == 0;
+  float m = has_sink ? sinks[head] * 1.4426950408889634f : -INFINITY;
+  const float l0 = has_sink ? 1.f : 0.f;
+  f32x4_t lsum = {l0, l0, l0, l0};   // the denominator of query column c, the same in all four places
   f32x4_t o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -951,7 +956,7 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
                                      const int* positions, const int* cu_seqlens, const int* block_table,
                                      int table_width, const void* kcache, const void* vcache, int page_size,
                                      int n_seqs, int max_new, int nh, int nkv, int hd, float scale, int window,
-                                     int queries, hipStream_t stream) {
+                                     int queries, const float* sinks, hipStream_t stream) {
   BLM_REQUIRE(n_seqs > 0 && n_seqs <= 65535 && max_new > 0 && nh > 0 && nkv > 0 && nkv <= 65535 && nh % nkv == 0,
               "attn_prefill_mfma: bad sizes seqs=%d max_new=%d heads=%d kv_heads=%d", n_seqs, max_new, nh, nkv);
   BLM_REQUIRE(blm_attn_prefill_mfma_supported(act_dtype, hd, page_size),
@@ -979,7 +984,7 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
   case HD:                                                                                                       \
     hipLaunchKernelGGL((attn_prefill32_kernel<HD>), grid32, block32, 0, stream, (const bf16*)q, q_row_stride,     \
                        (bf16*)out, positions, cu_seqlens, block_table, table_width, (const bf16*)kcache,          \
-                       (const bf16*)vcache, nh, nkv, scale, window);                                              \
+                       (const bf16*)vcache, nh, nkv, scale, window, sinks);                                       \
     break
     switch (hd) {
       BLM_AP32(32); BLM_AP32(64); BLM_AP32(96); BLM_AP32(128);
@@ -994,7 +999,7 @@ extern "C" int blm_attn_prefill_mfma(const void* q, int q_row_stride, void* out,
   case HD:                                                                                                       \
     hipLaunchKernelGGL((attn_prefill_mfma_kernel<HD>), grid, block, 0, stream, (const bf16*)q, q_row_stride,      \
                        (bf16*)out, positions, cu_seqlens, block_table, table_width, (const bf16*)kcache,          \
-                       (const bf16*)vcache, nh, nkv, scale, window);                                              \
+                       (const bf16*)vcache, nh, nkv, scale, window, sinks);                                       \
     break
   switch (hd) {
     BLM_AP(16); BLM_AP(32); BLM_AP(48); BLM_AP(64); BLM_AP(80); BLM_AP(96); BLM_AP(112); BLM_AP(128); BLM_AP(256);
@@ -1011,7 +1016,7 @@ extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int a
                                const int* token_seq, const int* block_table, int table_width, const void* kcache,
                                const void* vcache, int page_size, int T, int nh, int nkv, int hd, float scale,
                                int window, int n_splits, float* part_o, float* part_ml, int* arrivals,
-                               hipStream_t stream) {
+                               const float* sinks, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && T <= 65535 && nh > 0 && nkv > 0 && nh % nkv == 0,
               "attn_decode: bad sizes T=%d heads=%d kv_heads=%d", T, nh, nkv);
   BLM_REQUIRE(blm_attn_decode_supported(act_dtype, hd, page_size),
@@ -1031,7 +1036,7 @@ extern "C" int blm_attn_decode(const void* q, int q_row_stride, void* out, int a
   case HD:                                                                                                         \
     hipLaunchKernelGGL((attn_decode_mfma_kernel<HD>), grid, block, 0, stream, (const bf16*)q, q_row_stride,         \
                        positions, token_seq, block_table, table_width, (const bf16*)kcache, (const bf16*)vcache,    \
-                       nh, nkv, scale, window, n_splits, part_o, part_ml, arrivals, (bf16*)out);                    \
+                       nh, nkv, scale, window, n_splits, part_o, part_ml, arrivals, (bf16*)out, sinks);             \
     break
   switch (hd) { BLM_AD(16); BLM_AD(32); BLM_AD(48); BLM_AD(64); BLM_AD(80); BLM_AD(96); BLM_AD(112); BLM_AD(128); }
 #undef BLM_AD

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 34
+ABI_VERSION = 35
 _lib = None
 _lock = threading.Lock()
 
@@ -85,12 +85,12 @@ _SIGNATURES = {
                        _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
     "blm_attn_decode": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int,
-                        _c_void_p, _c_void_p, _c_void_p, _c_void_p],
+                        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p],
     "blm_attn_decode_supported": [_c_int, _c_int, _c_int],
     "blm_attn_prefill_mfma_supported": [_c_int, _c_int, _c_int],
     "blm_attn_prefill_mfma": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                               _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                              _c_int, _c_int, _c_void_p],
+                              _c_int, _c_int, _c_void_p, _c_void_p],
     "blm_gemm_tiled": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_void_p],
     "blm_gemv_skinny": [_c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
@@ -386,11 +386,14 @@ def attn_prefill_queries(n_seqs, max_new, nh, nkv, hd, compute_units):
 
 
 def attn_prefill_mfma(q, q_row_stride, out, positions, cu_seqlens, block_table, kcache, vcache, page_size,
-                      n_seqs, max_new, nh, nkv, hd, scale, window=0, queries=16):
+                      n_seqs, max_new, nh, nkv, hd, scale, window=0, queries=16, sinks=None):
     """Causal attention of packed sequences over their cached keys on the matrix cores (bfloat16).
     Rows cu_seqlens[b] .. cu_seqlens[b+1] of q and out belong to sequence b; max_new is the most
-    rows any sequence has.  queries: 16 or 32 query rows per wavefront (attn_prefill_queries chooses)."""
-    _gpu(q, out, positions, cu_seqlens, block_table, kcache, vcache)
+    rows any sequence has.  queries: 16 or 32 query rows per wavefront (attn_prefill_queries chooses).
+    sinks (float32 [heads]): the softmax's denominator also holds exp(sinks[h]), a logit without key or value."""
+    _gpu(q, out, positions, cu_seqlens, block_table, kcache, vcache, sinks)
+    if sinks is not None:
+        _f32("sinks", sinks, nh)
     T = out.shape[0]
     _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache)
     if out.shape[1] != nh * hd or out.dtype != q.dtype or kcache.dtype != q.dtype:
@@ -403,14 +406,17 @@ def attn_prefill_mfma(q, q_row_stride, out, positions, cu_seqlens, block_table, 
         raise KernelError("attn_prefill_mfma: the page table has fewer rows than there are sequences")
     _call("blm_attn_prefill_mfma", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
           cu_seqlens.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
-          page_size, int(n_seqs), int(max_new), nh, nkv, hd, float(scale), int(window), int(queries), _stream())
+          page_size, int(n_seqs), int(max_new), nh, nkv, hd, float(scale), int(window), int(queries), _ptr(sinks), _stream())
     return out
 
 
 def attn_decode(q, q_row_stride, out, positions, token_seq, block_table, kcache, vcache, page_size,
-                nh, nkv, hd, scale, window=0, n_splits=1):
-    """Attention for few query tokens over long key ranges, the key range cut into n_splits."""
-    _gpu(q, out, positions, token_seq, block_table, kcache, vcache)
+                nh, nkv, hd, scale, window=0, n_splits=1, sinks=None):
+    """Attention for few query tokens over long key ranges, the key range cut into n_splits.  sinks: as for
+    attn_prefill_mfma."""
+    _gpu(q, out, positions, token_seq, block_table, kcache, vcache, sinks)
+    if sinks is not None:
+        _f32("sinks", sinks, nh)
     T = out.shape[0]
     _contig("out", out); _contig("kcache", kcache); _contig("vcache", vcache)
     if out.shape[1] != nh * hd or out.dtype != q.dtype or kcache.dtype != q.dtype:
@@ -428,7 +434,7 @@ def attn_decode(q, q_row_stride, out, positions, token_seq, block_table, kcache,
     _call("blm_attn_decode", q.data_ptr(), q_row_stride, out.data_ptr(), _code(out), positions.data_ptr(),
           token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], kcache.data_ptr(), vcache.data_ptr(),
           page_size, T, nh, nkv, hd, float(scale), int(window), n_splits, _ptr(part_o), _ptr(part_ml),
-          _ptr(arrivals), _stream())
+          _ptr(arrivals), _ptr(sinks), _stream())
     return out
 
 

@@ -94,6 +94,11 @@ class SinkAttention(Mixer):
         self.output_bias = tensors[n["o_bias"]].float().contiguous() if bias else None
         self.on_matrix_cores = rt.ops.sink_attn_mfma_supported(rt.dtype, self.dk, self.dv) and self.scale > 0 \
             and os.environ.get("BURN_LM_AMD_SINK_ATTENTION") != "generic"
+        # without head mixing and with values of the keys' size this is the plain attention's arithmetic plus a share of
+        # the denominator: the plain attention's matrix-core kernels take the sink
+        self.on_plain_kernels = self.on_matrix_cores and not talk and self.dk == self.dv \
+            and rt.ops.attn_decode_supported(rt.dtype, self.dk) and rt.ops.attn_prefill_mfma_supported(rt.dtype, self.dk) \
+            and os.environ.get("BURN_LM_AMD_SINK_ATTENTION") != "own"
         if self.on_matrix_cores:
             rt.ops.latent_attn_init(rt.device)     # the pieces' workspace, before any step is recorded
             rt.ops.sink_attn_mfma_init(rt.device)  # likewise: the shared memory of the form that stages pages
@@ -149,6 +154,8 @@ class SinkAttention(Mixer):
         brings so few tiles (decoding) that they would leave most of the chip idle; else the generic kernel."""
         rt = self.rt
         out = torch.empty(qkv.shape[0], self.H * self.dv, dtype=rt.dtype, device=qkv.device)
+        if self.on_plain_kernels and view.page_size == 64 and qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0:
+            return self._attend_plain(qkv, out, step, view)
         if self.on_matrix_cores and view.page_size == 64 and qkv.stride(0) % 8 == 0 and qkv.data_ptr() % 16 == 0 \
                 and hasattr(step, "lens_after"):
             n_splits, group_batch = 1, 0
@@ -166,6 +173,27 @@ class SinkAttention(Mixer):
                                          n_splits=n_splits, group_batch=group_batch)
         return rt.ops.sink_attn(qkv, out, self.sinks, self.talk, step, view.block_table(step), view.k, view.v,
                                 view.page_size, self.H, self.G, self.dk, self.dv, self.scale, self.window)
+
+    def _attend_plain(self, qkv, out, step, view):
+        """The plain attention's kernels (decode: key ranges cut as that mixer cuts them), with the sink."""
+        from .attention import decode_splits
+        rt, table = self.rt, view.block_table(step)
+        H, G, hd = self.H, self.G, self.dk
+        if step.max_new == 1:
+            span = step.max_len_after if not self.window else min(step.max_len_after, self.window + view.page_size)
+            pages = (span + view.page_size - 1) // view.page_size
+            blocks = qkv.shape[0] * G * ((H // G + 15) // 16)
+            rt.ops.attn_decode(qkv, qkv.stride(0), out, step.positions, step.token_seq, table, view.k, view.v, view.page_size,
+                               H, G, hd, self.scale, self.window, decode_splits(pages, blocks, hd, rt.compute_units),
+                               sinks=self.sinks)
+        else:
+            queries = rt.prefill_queries or rt.ops.attn_prefill_queries(step.n_seqs, step.max_new, H, G, hd, rt.compute_units)
+            if queries == 32 and (hd % 32 or hd > 128):
+                queries = 16
+            rt.ops.attn_prefill_mfma(qkv, qkv.stride(0), out, step.positions, step.cu_seqlens, table, view.k, view.v,
+                                     view.page_size, step.n_seqs, step.max_new, H, G, hd, self.scale, self.window,
+                                     queries=queries, sinks=self.sinks)
+        return out
 
     def output(self, attended):
         return self.rt.linear(attended, self.w_o, partials=True)

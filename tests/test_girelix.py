@@ -429,15 +429,25 @@ class _Step:
 
 
 def _attend(form, *args):
-    """The generic kernel, or the matrix-core one with its pages whole or cut into pieces."""
+    """The generic kernel, the matrix-core one with its pages whole or cut into pieces, or the plain attention's
+    kernels given the sink (16 or 32 queries per wavefront in prompts, key ranges whole or cut in decoding)."""
     from burn_lm_amd.csrc import ops
     if form == "generic":
         return ops.sink_attn(*args)
+    if form.startswith("plain"):
+        q, out, sinks, mix, step, table, kc, vc, ps, H, G, dk, dv, scale, window = args
+        assert mix is None and dk == dv
+        if step.max_new == 1:
+            return ops.attn_decode(q, q.stride(0), out, step.positions, step.token_seq, table, kc, vc, ps, H, G, dk, scale,
+                                   window, n_splits=3 if form == "plain_cut" else 1, sinks=sinks)
+        return ops.attn_prefill_mfma(q, q.stride(0), out, step.positions, step.cu_seqlens, table, kc, vc, ps, step.n_seqs,
+                                     step.max_new, H, G, dk, scale, window, queries=32 if form == "plain_cut" else 16, sinks=sinks)
     return ops.sink_attn_mfma(*args, n_splits=1 if form == "matrix" else 3, group_batch=0 if form == "matrix" else 1)
 
 
-FORMS = [("generic", torch.float32), ("generic", torch.bfloat16), ("matrix", torch.bfloat16), ("matrix_pieces", torch.bfloat16)]
-FORM_IDS = ["generic-float32", "generic-bfloat16", "matrix", "matrix_pieces"]
+FORMS = [("generic", torch.float32), ("generic", torch.bfloat16), ("matrix", torch.bfloat16), ("matrix_pieces", torch.bfloat16),
+         ("plain", torch.bfloat16), ("plain_cut", torch.bfloat16)]
+FORM_IDS = ["generic-float32", "generic-bfloat16", "matrix", "matrix_pieces", "plain", "plain_cut"]
 
 
 @pytest.mark.gpu
@@ -448,7 +458,7 @@ def test_one_key_far_back_among_hundreds_and_the_sink(form, dtype, decode):
     value wherever the key lies (the first token, the last and first places of pages that lie scattered), and must not
     know it before the query reaches it.  Then the sink towers over all keys, and the result must be nothing."""
     dev = "cuda"
-    H, G, dk, ps = 4, 2, 8, 64
+    H, G, dk, ps = 4, 2, (32 if form.startswith("plain") else 8), 64
     g = torch.Generator().manual_seed(0)
     pages = [7, 2, 5, 0, 8, 3]                                   # the sequence's pages; pages 1, 4, 6 hold noise
     kc = torch.randn(9, G, ps, dk, generator=g) * 0.1
