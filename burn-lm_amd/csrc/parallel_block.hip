@@ -520,14 +520,15 @@ extern "C" int blm_scaled_add(float* h, int T, int D, int n_terms,
 #define PB_MAX_ROUTED 256
 #define PB_ROUTED_PER_LANE (PB_MAX_ROUTED / BLM_WAVE)
 
-// the largest (value, index) pair over a wavefront; of equal values the one with the lower index
+// the largest (value, index) pair over a wavefront; of equal values the one with the lower index (indices below 2^24;
+// 0x7fffffff stands for "none").  Two reductions across lanes instead of a pair that travels: first the value, then the
+// smallest index among the lanes that hold it.
 __device__ __forceinline__ void pb_wave_best(float& v, int& i) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    const float ov = __shfl_xor(v, off);
-    const int oi = __shfl_xor(i, off);
-    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
-  }
+  const float best = wave_max(v);
+  const float mine = (v == best && i != 0x7fffffff) ? -(float)i : -3.0e9f;
+  const float first = -wave_max(mine);
+  v = best;
+  i = first < 2.0e9f ? (int)first : 0x7fffffff;
 }
 
 // One wavefront per token; lane l holds the experts l, l + 64, ...  Scores and corrected scores stay in registers; the
