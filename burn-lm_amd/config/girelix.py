@@ -3,8 +3,8 @@
 Top level: ``vocab``, ``width``, ``norm.eps``, ``residual_mult`` and ``layers``: a list of ``{type, mixer, mlp}``.
 ``type`` is ``parallel``: one norm whose output the mixer and the feed-forward both read.  ``mixer`` holds two mixers
 side by side, ``left`` (softmax attention: ``heads, kv_heads, dim, vdim, scale, rot: {dims, base}``) and ``right``
-(lightning attention: ``heads, dim, vdim, decay`` with one decay per head), and their factors ``left_scale`` and
-``right_scale``.  ``mlp`` is ``null`` (none) or ``{kind: moe, expert: {ff}, router: {experts, top, identity,
+(lightning attention: ``heads, dim, vdim, decay`` with one decay per head, or one number for all), and their factors
+``left_scale`` and ``right_scale``.  ``mlp`` is ``null`` (none) or ``{kind: moe, expert: {ff}, router: {experts, top, identity,
 groups: {count, keep}}}`` (``identity`` and ``groups`` may be missing: no pass-through experts, one group).  Every
 size is a required key."""
 from __future__ import annotations
@@ -118,6 +118,8 @@ class GirelixConfig:
             r, rw = m.get("right"), mw + ".right"
             r_heads = _get(r, "heads", int, rw)
             decay = r.get("decay")
+            if isinstance(decay, (int, float)) and not isinstance(decay, bool):
+                decay = [decay] * r_heads      # one number for all heads
             if not isinstance(decay, list) or len(decay) != r_heads \
                     or not all(isinstance(a, (int, float)) and not isinstance(a, bool) and 0.0 < a <= 1.0 for a in decay):
                 raise ConfigError(f"config.json: {rw}.decay must list one number in (0, 1] for each of the {r_heads} heads")

@@ -156,6 +156,9 @@ def test_config_is_read_and_refused_by_key():
         at[path[-1]] = value
         with pytest.raises(ConfigError, match=word):
             arch.read_config(bad)
+    one = json.loads(json.dumps(MIXED))
+    one["layers"][0]["mixer"]["right"]["decay"] = 0.75      # one number stands for every head
+    assert arch.read_config(one).layers[0].mixer.right.decay == (0.75,) * one["layers"][0]["mixer"]["right"]["heads"]
 
 
 def test_plan_asks_for_the_checkpoints_tensors():
@@ -365,7 +368,7 @@ def drawn_config(seed):
     pick = lambda *a: a[int(rng.integers(0, len(a)))]
     layers = []
     for _ in range(int(rng.integers(1, 5))):
-        G, dk = int(rng.integers(1, 4)), pick(8, 16, 24, 32, 48, 64, 12, 6)
+        G, dk = int(rng.integers(1, 4)), pick(8, 16, 24, 32, 48, 64, 12, 6, 80, 96, 128)
         rh = int(rng.integers(1, 5))
         if rng.random() < 0.25:
             mlp = None
@@ -379,9 +382,9 @@ def drawn_config(seed):
             mlp = moe(experts=n - identity, identity=identity, top=int(rng.integers(1, room + 1)), count=count, keep=keep,
                       ff=pick(8, 16, 40, 6))
         layers.append(layer(heads=G * int(rng.integers(1, 5)), kv_heads=G, dim=dk,
-                            rot=pick(0, *[d for d in (2, 4, 6, 8, 12, 16, 24, 32, 48, 64) if d <= dk]),
+                            rot=pick(0, *[d for d in (2, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128) if d <= dk]),
                             base=pick(100.0, 10000.0, 5e5), scale=pick(0.1, 0.25, 0.5), r_heads=rh,
-                            r_dim=pick(8, 16, 24, 48, 5), r_vdim=pick(8, 16, 32, 20, 3),
+                            r_dim=pick(8, 16, 24, 48, 5, 64, 128), r_vdim=pick(8, 16, 32, 20, 3, 64, 128),
                             decay=[pick(0.3, 0.8, 0.95, 0.99, 0.999, 1.0) for _ in range(rh)],
                             left_scale=pick(0.5, 1.0, 1.5), right_scale=pick(0.5, 1.0, 1.5), mlp=mlp))
     return config(layers, width=pick(40, 64, 96, 128, 72), vocab=pick(50, 101, 257), mult=pick(0.5, 1.0, 1.4), eps=pick(1e-5, 1e-6))
@@ -389,7 +392,7 @@ def drawn_config(seed):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16])
+@pytest.mark.parametrize("seed", [11, 12, 13, 14, 15, 16, 17, 18])
 def test_drawn_configurations(tmp_path, seed, dtype):
     """Unequal prompts in one step, then 32 tokens one by one, for configurations nobody chose by hand."""
     cfg = drawn_config(seed)
