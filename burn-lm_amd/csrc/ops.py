@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 35
+ABI_VERSION = 36
 _lib = None
 _lock = threading.Lock()
 
@@ -38,6 +38,11 @@ _SIGNATURES = {
     "blm_gla_scan": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_float, _c_void_p, _c_void_p,
                      _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                      _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_float, _c_int, _c_int, _c_void_p],
+    "blm_lightning_chunks_init": [],
+    "blm_lightning_chunks_supported": [_c_int, _c_int],
+    "blm_lightning_chunks": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                             _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                             _c_int, _c_int, _c_int, _c_void_p],
     "blm_qkv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                         _c_void_p],
@@ -1301,6 +1306,57 @@ def gla_scan(proj, decay_in, decay_bias, tau, norm_w, eps, state, o_raw, out, st
           seg_len, _ptr(seg_end), _ptr(seg_start), _ptr(seg_decay), _ptr(q_tilde), _ptr(fixed_decay),
           1 if activation == "silu" else 0, float(q_scale) if q_scale is not None else 0.0, 1 if norm_all else 0,
           GATE_MODES[gate], _stream())
+    return out
+
+
+LIGHTNING_CHUNK = 64
+_lc_ready = set()
+
+
+def lightning_chunks_init(device=None):
+    """Once per device, outside any stream capture, before the first lightning_chunks (its kernels take more shared
+    memory than a kernel gets without asking)."""
+    index = torch.device(device or "cuda").index
+    index = torch.cuda.current_device() if index is None else index
+    if index not in _lc_ready:
+        with torch.cuda.device(index):
+            _call("blm_lightning_chunks_init")
+        _lc_ready.add(index)
+
+
+def lightning_chunks_supported(dk, dv):
+    return bool(library().blm_lightning_chunks_supported(int(dk), int(dv)))
+
+
+def decay_powers(decays, device):
+    """float32 [heads, 65]: powers 0 .. 64 of every head's decay, from double precision."""
+    a = torch.tensor([float(x) for x in decays], dtype=torch.float64).reshape(-1, 1)
+    return (a ** torch.arange(LIGHTNING_CHUNK + 1, dtype=torch.float64)).to(torch.float32).contiguous().to(device)
+
+
+def lightning_chunks(proj, powers, norm_w, eps, state, o_raw, out, step, H, dk, dv, activation=None, norm_all=False,
+                     gate="sigmoid"):
+    """Linear attention with one constant decay per head over the prompts of a step, in chunks of 64 tokens as float32
+    matrix products: proj [T, >= 2 H dk + 2 H dv] (queries, keys, values, output-gate logits; not changed), powers as
+    decay_powers gives them, state float32 [slots, H, dk, dv] read and left updated, o_raw float32 [T, H * dv], out
+    [T, H * dv] in proj's dtype.  activation, norm_all, gate as for gla_scan; the queries have no factor."""
+    _gpu(proj, powers, norm_w, state, o_raw, out)
+    T = proj.shape[0]
+    _f32("o_raw", o_raw, T * H * dv); _f32("norm_w", norm_w, H * dv if norm_all else dv); _f32("state", state)
+    _f32("powers", powers, H * (LIGHTNING_CHUNK + 1)); _contig("out", out)
+    if activation not in (None, "silu") or gate not in GATE_MODES:
+        raise KernelError(f"lightning_chunks: activation {activation!r} or gate {gate!r} unknown")
+    if proj.stride(1) != 1 or out.dtype != proj.dtype or tuple(out.shape) != (T, H * dv) or tuple(state.shape[1:]) != (H, dk, dv) \
+            or proj.shape[1] < 2 * H * dk + 2 * H * dv or T != step.n_tokens:
+        raise KernelError("lightning_chunks: shapes do not fit")
+    B, n_seg = step.n_seqs, -(-step.max_new // LIGHTNING_CHUNK)
+    seg_end = torch.empty(B, n_seg, H, dk, dv, dtype=torch.float32, device=proj.device)
+    seg_start = torch.empty_like(seg_end)
+    seg_decay = torch.empty(B, n_seg, H, dk, dtype=torch.float32, device=proj.device)
+    _call("blm_lightning_chunks", proj.data_ptr(), _code(proj), proj.stride(0), powers.data_ptr(), norm_w.data_ptr(), float(eps),
+          state.data_ptr(), o_raw.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, B, H, dk,
+          dv, step.max_new, n_seg, seg_end.data_ptr(), seg_start.data_ptr(), seg_decay.data_ptr(),
+          1 if activation == "silu" else 0, 1 if norm_all else 0, GATE_MODES[gate], _stream())
     return out
 
 

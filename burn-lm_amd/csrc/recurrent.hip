@@ -936,3 +936,291 @@ extern "C" int blm_gla_scan(void* proj, int dtype, int ld, const void* decay_in,
   if (norm_all) return launch_head_norm(o_raw, norm_w, gate, ld, gate_mode, 1, out, dtype, (long long)T, H * dv, eps, stream);
   return launch_head_norm(o_raw, norm_w, gate, ld, gate_mode, H, out, dtype, (long long)T * H, dv, eps, stream);
 }
+
+// ---------------------------------------------------------------------------------------
+// Lightning attention over prompts: chunks of 64 tokens as float32 matrix products.
+// With ONE constant decay a per head the recurrence S_t = a S_(t-1) + k_t v_t^T, o_t = S_t^T q_t has a closed form inside
+// a chunk of n tokens that starts from the state S0 (i, j count from the chunk's first token):
+//   O = (Q K^T * L) V + diag(a^(i+1)) Q S0,   L_ij = a^(i-j) for j <= i, else 0
+//   S_end = a^n S0 + (diag(a^(n-1-j)) K)^T V
+// All powers are at most one and come from a table pw [H][65] = a^0 .. a^64 (made in double precision), so no quotient or
+// running product of decays appears and a fast decay cannot overflow.  Three kernels: lc_state (every chunk's own
+// contribution (diag(..) K)^T V, the first chunk's with the sequence's state), gla_carry (the chunks' start states in
+// order, and the sequence's new state), lc_out (the chunk's results).  Operands are staged through shared memory in the
+// rows' type (the activated queries, keys and values are rounded to it, as a projection's output is) and multiplied by
+// 32x32x2 float32 matrix instructions: lane l holds row l % 32 of the left operand and column l % 32 of the right one at
+// depth l / 32; result register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
+// Heads of up to 128 key and 128 value channels, padded to multiples of 32 with zeros.
+// ---------------------------------------------------------------------------------------
+#define LC_CHUNK 64
+#define LC_MAX 128
+#define LC_THREADS 256
+#define LC_A_LD (LC_CHUNK + 1)
+#define LC_LDS_LIMIT (128 * 1024)
+typedef float lc_acc __attribute__((ext_vector_type(16)));
+
+template <typename TA>
+__device__ __forceinline__ int lc_row_pad() { return sizeof(TA) == 4 ? 1 : 2; }      // an odd number of 4-byte words per row
+
+template <typename TA>
+__device__ __forceinline__ float lc_read(const TA* __restrict__ p, int act) {
+  const float x = to_float(*p);
+  return act ? to_float(from_float<TA>(blm_silu(x))) : x;
+}
+
+// seg_end [B][n_seg][H][dk][dv], seg_start likewise (only chunk 0 is written here), seg_decay [B][n_seg][H][dk]
+template <typename TA>
+__global__ void __launch_bounds__(LC_THREADS)
+    lc_state_kernel(const TA* __restrict__ proj, int ld, int act, const float* __restrict__ pw, const float* __restrict__ state,
+                    float* __restrict__ seg_end, float* __restrict__ seg_start, float* __restrict__ seg_decay,
+                    const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk, int dv, int n_seg) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lc_sm[];
+  const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int slot = seq_slots[b], first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - first;
+  const int t0 = c * LC_CHUNK;
+  if (slot < 0 || t0 >= n_new) return;
+  const int n = min(LC_CHUNK, n_new - t0);
+  const int DKP = (dk + 31) & ~31, DVP = (dv + 31) & ~31;
+  float* Kf = reinterpret_cast<float*>(lc_sm);                      // [64][DKP], each key times a^(n-1-j)
+  TA* Vs = reinterpret_cast<TA*>(Kf + LC_CHUNK * DKP);              // [64][DVP]
+  const float* pwh = pw + h * (LC_CHUNK + 1);
+  const TA* rows = proj + (size_t)(first + t0) * ld;
+  for (int e = threadIdx.x; e < LC_CHUNK * DKP; e += LC_THREADS) {
+    const int j = e / DKP, i = e - j * DKP;
+    Kf[e] = (j < n && i < dk) ? lc_read(rows + (size_t)j * ld + (size_t)H * dk + h * dk + i, act) * pwh[n - 1 - j] : 0.f;
+  }
+  for (int e = threadIdx.x; e < LC_CHUNK * DVP; e += LC_THREADS) {
+    const int j = e / DVP, i = e - j * DVP;
+    Vs[e] = from_float<TA>((j < n && i < dv) ? lc_read(rows + (size_t)j * ld + (size_t)2 * H * dk + h * dv + i, act) : 0.f);
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int lr = lane & 31, lk = lane >> 5;
+  const int NV = DVP / 32, tiles = (DKP / 32) * NV;
+  const int depth = (n + 1) & ~1;
+  lc_acc acc[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[s][r] = 0.f;
+  for (int k0 = 0; k0 < depth; k0 += 2) {
+    const float* krow = Kf + (k0 + lk) * DKP + lr;
+    const TA* vrow = Vs + (k0 + lk) * DVP + lr;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int t = wave + 4 * s;
+      if (t < tiles) {
+        const int tr = t / NV, tc = t - tr * NV;
+        acc[s] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[tr * 32], to_float(vrow[tc * 32]), acc[s], 0, 0, 0);
+      }
+    }
+  }
+  const size_t per = (size_t)dk * dv;
+  const size_t at = (((size_t)b * n_seg + c) * H + h) * per;
+  const float* S_old = state + ((size_t)slot * H + h) * per;
+  const float fade = pwh[n];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int t = wave + 4 * s;
+    if (t < tiles) {
+      const int tr = t / NV, tc = t - tr * NV;
+      const int col = tc * 32 + lr;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = tr * 32 + 8 * (r / 4) + 4 * lk + (r & 3);
+        if (i < dk && col < dv) {
+          float v = acc[s][r];
+          if (c == 0) {
+            const float old = S_old[(size_t)i * dv + col];
+            seg_start[at + (size_t)i * dv + col] = old;
+            v = fmaf(fade, old, v);
+          }
+          seg_end[at + (size_t)i * dv + col] = v;
+        }
+      }
+    }
+  }
+  for (int i = threadIdx.x; i < dk; i += LC_THREADS) seg_decay[(((size_t)b * n_seg + c) * H + h) * dk + i] = fade;
+}
+
+template <typename TA>
+__global__ void __launch_bounds__(LC_THREADS)
+    lc_out_kernel(const TA* __restrict__ proj, int ld, int act, const float* __restrict__ pw, const float* __restrict__ seg_start,
+                  float* __restrict__ o_raw, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk,
+                  int dv, int n_seg) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lc_sm[];
+  const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int slot = seq_slots[b], first = cu_seqlens[b], n_new = cu_seqlens[b + 1] - first;
+  const int t0 = c * LC_CHUNK;
+  if (slot < 0 || t0 >= n_new) return;
+  const int n = min(LC_CHUNK, n_new - t0);
+  const int DKP = (dk + 31) & ~31, DVP = (dv + 31) & ~31;
+  const int SK = DKP + lc_row_pad<TA>();
+  float* As = reinterpret_cast<float*>(lc_sm);                      // [64][65]: (Q K^T) * L
+  float* pws = As + LC_CHUNK * LC_A_LD;                             // [65] (+ 3 unused)
+  TA* Qs = reinterpret_cast<TA*>(pws + LC_CHUNK + 4);               // [64][SK]
+  TA* Ks = Qs + LC_CHUNK * SK;                                      // [64][SK]
+  TA* Vs = Ks + LC_CHUNK * SK;                                      // [64][DVP]
+  const TA* rows = proj + (size_t)(first + t0) * ld;
+  for (int e = threadIdx.x; e < LC_CHUNK * DKP; e += LC_THREADS) {
+    const int j = e / DKP, i = e - j * DKP;
+    const bool in = j < n && i < dk;
+    Qs[j * SK + i] = from_float<TA>(in ? lc_read(rows + (size_t)j * ld + h * dk + i, act) : 0.f);
+    Ks[j * SK + i] = from_float<TA>(in ? lc_read(rows + (size_t)j * ld + (size_t)H * dk + h * dk + i, act) : 0.f);
+  }
+  for (int e = threadIdx.x; e < LC_CHUNK * DVP; e += LC_THREADS) {
+    const int j = e / DVP, i = e - j * DVP;
+    Vs[e] = from_float<TA>((j < n && i < dv) ? lc_read(rows + (size_t)j * ld + (size_t)2 * H * dk + h * dv + i, act) : 0.f);
+  }
+  if (threadIdx.x <= LC_CHUNK) pws[threadIdx.x] = pw[h * (LC_CHUNK + 1) + threadIdx.x];
+  __syncthreads();
+  const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
+  const int lr = lane & 31, lk = lane >> 5;
+  const int depth_k = (dk + 1) & ~1;
+  // scores of the three tiles at and below the diagonal, times the powers of the decay
+  if (wave < 3) {
+    const int ti = wave == 0 ? 0 : 1, tj = wave == 2 ? 1 : 0;
+    lc_acc sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+    const TA* qrow = Qs + (ti * 32 + lr) * SK + lk;
+    const TA* krow = Ks + (tj * 32 + lr) * SK + lk;
+#pragma unroll 4
+    for (int k0 = 0; k0 < depth_k; k0 += 2)
+      sc = __builtin_amdgcn_mfma_f32_32x32x2f32(to_float(qrow[k0]), to_float(krow[k0]), sc, 0, 0, 0);
+    const int j = tj * 32 + lr;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = ti * 32 + 8 * (r / 4) + 4 * lk + (r & 3);
+      As[i * LC_A_LD + j] = j <= i ? sc[r] * pws[i - j] : 0.f;
+    }
+  }
+  __syncthreads();
+  const int NV = DVP / 32;
+  const int ti = wave & 1, tc0 = wave >> 1;
+  lc_acc acc[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[s][r] = 0.f;
+  // what the chunk's start state gives: Q S0, row i times a^(i+1)
+  {
+    const float* S0 = seg_start + (((size_t)b * n_seg + c) * H + h) * (size_t)dk * dv;
+    const TA* qrow = Qs + (ti * 32 + lr) * SK + lk;
+    const int col0 = tc0 * 32 + lr, col1 = (tc0 + 2) * 32 + lr;
+    const bool in0 = tc0 < NV && col0 < dv, in1 = tc0 + 2 < NV && col1 < dv;
+#pragma unroll 4
+    for (int k0 = 0; k0 < depth_k; k0 += 2) {
+      const int kk = k0 + lk;
+      const float a = to_float(qrow[k0]);
+      const float s0 = (in0 && kk < dk) ? S0[(size_t)kk * dv + col0] : 0.f;
+      const float s1 = (in1 && kk < dk) ? S0[(size_t)kk * dv + col1] : 0.f;
+      if (tc0 < NV) acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s0, acc[0], 0, 0, 0);
+      if (tc0 + 2 < NV) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s1, acc[1], 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float f = pws[ti * 32 + 8 * (r / 4) + 4 * lk + (r & 3) + 1];
+      acc[0][r] *= f;
+      acc[1][r] *= f;
+    }
+  }
+  // what the chunk's own tokens give: (scores * L) V, over the keys up to the row tile's last row
+  {
+    const float* arow = As + (ti * 32 + lr) * LC_A_LD + lk;
+    const TA* vrow = Vs + lk * DVP + lr;
+    const int depth = min((ti + 1) * 32, (n + 1) & ~1);
+#pragma unroll 4
+    for (int k0 = 0; k0 < depth; k0 += 2) {
+      const float a = arow[k0];
+      if (tc0 < NV) acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(vrow[k0 * DVP + tc0 * 32]), acc[0], 0, 0, 0);
+      if (tc0 + 2 < NV) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(vrow[k0 * DVP + (tc0 + 2) * 32]), acc[1], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int tc = tc0 + 2 * s;
+    const int col = tc * 32 + lr;
+    if (tc < NV && col < dv) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = ti * 32 + 8 * (r / 4) + 4 * lk + (r & 3);
+        if (i < n) o_raw[((size_t)(first + t0 + i) * H + h) * dv + col] = acc[s][r];
+      }
+    }
+  }
+}
+
+static size_t lc_state_lds(int dk, int dv, int dtype) {
+  const int DKP = (dk + 31) & ~31, DVP = (dv + 31) & ~31;
+  return (size_t)LC_CHUNK * DKP * sizeof(float) + (size_t)LC_CHUNK * DVP * (dtype == BLM_F32 ? 4 : 2);
+}
+static size_t lc_out_lds(int dk, int dv, int dtype) {
+  const int DKP = (dk + 31) & ~31, DVP = (dv + 31) & ~31;
+  const int es = dtype == BLM_F32 ? 4 : 2, SK = DKP + (dtype == BLM_F32 ? 1 : 2);
+  return (size_t)(LC_CHUNK * LC_A_LD + LC_CHUNK + 4) * sizeof(float) + (size_t)LC_CHUNK * (2 * SK + DVP) * es;
+}
+
+#define LC_DEVICES 64
+static bool g_lc_ready[LC_DEVICES];
+// Once per device, outside any stream capture: the chunk kernels take more shared memory than a kernel gets without asking.
+extern "C" int blm_lightning_chunks_init() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  BLM_REQUIRE(e == hipSuccess && dev >= 0 && dev < LC_DEVICES, "lightning_chunks_init: hipGetDevice failed or device %d is beyond %d", dev, LC_DEVICES);
+  const void* ks[] = {(const void*)lc_state_kernel<float>, (const void*)lc_state_kernel<bf16>, (const void*)lc_out_kernel<float>,
+                      (const void*)lc_out_kernel<bf16>};
+  for (const void* k : ks) {
+    e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, LC_LDS_LIMIT);
+    BLM_REQUIRE(e == hipSuccess, "lightning_chunks_init: cannot raise the shared memory limit: %s", hipGetErrorString(e));
+  }
+  g_lc_ready[dev] = true;
+  return 0;
+}
+
+extern "C" int blm_lightning_chunks_supported(int dk, int dv) { return (dk >= 1 && dk <= LC_MAX && dv >= 1 && dv <= LC_MAX) ? 1 : 0; }
+
+// proj as for blm_gla_scan (queries, keys, values, output-gate logits); pw [H][65] float: powers 0 .. 64 of every head's
+// decay; n_seg: chunks of 64 tokens that cover the longest sequence of the step; seg_end, seg_start [B][n_seg][H][dk][dv],
+// seg_decay [B][n_seg][H][dk] float.  state is read and left updated; o_raw [T][H*dv] float; out [T][H*dv] in proj's type.
+// act_mode, norm_all, gate_mode as for blm_gla_scan (the activation happens on the way into shared memory: proj is not changed).
+extern "C" int blm_lightning_chunks(const void* proj, int dtype, int ld, const float* pw, const float* norm_w, float eps,
+                                    float* state, float* o_raw, void* out, const int* cu_seqlens, const int* seq_slots, int T,
+                                    int B, int H, int dk, int dv, int max_new, int n_seg, float* seg_end, float* seg_start,
+                                    float* seg_decay, int act_mode, int norm_all, int gate_mode, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && B > 0 && B <= 65535 && H > 0 && H <= 65535, "lightning_chunks: bad sizes T=%d B=%d H=%d", T, B, H);
+  BLM_REQUIRE(blm_lightning_chunks_supported(dk, dv), "lightning_chunks: heads of %d x %d channels are not supported (up to %d)", dk, dv, LC_MAX);
+  BLM_REQUIRE(ld >= 2 * H * dk + 2 * H * dv, "lightning_chunks: rows of %d are too short", ld);
+  BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "lightning_chunks: unsupported dtype %d", dtype);
+  BLM_REQUIRE(max_new >= 1 && n_seg >= 1 && (long long)n_seg * LC_CHUNK >= max_new && pw && seg_end && seg_start && seg_decay,
+              "lightning_chunks: %d chunks do not cover %d tokens, or no workspace", n_seg, max_new);
+  BLM_REQUIRE((act_mode == 0 || act_mode == 1) && (gate_mode == 1 || gate_mode == 2), "lightning_chunks: unknown activation %d or gate %d", act_mode, gate_mode);
+  int dev = -1;
+  BLM_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < LC_DEVICES && g_lc_ready[dev],
+              "lightning_chunks: blm_lightning_chunks_init has not run on device %d", dev);
+  const size_t lds_a = lc_state_lds(dk, dv, dtype), lds_c = lc_out_lds(dk, dv, dtype);
+  BLM_REQUIRE(lds_a <= LC_LDS_LIMIT && lds_c <= LC_LDS_LIMIT, "lightning_chunks: %zu bytes of shared memory are too many", lds_c);
+  const dim3 grid((unsigned)n_seg, (unsigned)H, (unsigned)B);
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(lc_state_kernel<float>, grid, dim3(LC_THREADS), lds_a, stream, (const float*)proj, ld, act_mode, pw, state,
+                       seg_end, seg_start, seg_decay, cu_seqlens, seq_slots, H, dk, dv, n_seg);
+  else
+    hipLaunchKernelGGL(lc_state_kernel<bf16>, grid, dim3(LC_THREADS), lds_a, stream, (const bf16*)proj, ld, act_mode, pw, state,
+                       seg_end, seg_start, seg_decay, cu_seqlens, seq_slots, H, dk, dv, n_seg);
+  BLM_LAUNCH_CHECK("lc_state");
+  const size_t per = (size_t)H * dk * dv;
+  const unsigned cb = (unsigned)((per + 255) / 256 < 1024 ? (per + 255) / 256 : 1024);
+  hipLaunchKernelGGL(gla_carry_kernel, dim3(cb, B), dim3(256), 0, stream, seg_end, seg_decay, seg_start, state, cu_seqlens,
+                     seq_slots, H, dk, dv, n_seg, LC_CHUNK);
+  BLM_LAUNCH_CHECK("gla_carry");
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(lc_out_kernel<float>, grid, dim3(LC_THREADS), lds_c, stream, (const float*)proj, ld, act_mode, pw, seg_start,
+                       o_raw, cu_seqlens, seq_slots, H, dk, dv, n_seg);
+  else
+    hipLaunchKernelGGL(lc_out_kernel<bf16>, grid, dim3(LC_THREADS), lds_c, stream, (const bf16*)proj, ld, act_mode, pw, seg_start,
+                       o_raw, cu_seqlens, seq_slots, H, dk, dv, n_seg);
+  BLM_LAUNCH_CHECK("lc_out");
+  const char* gate = (const char*)proj + (size_t)(2 * H * dk + H * dv) * (dtype == BLM_F32 ? 4 : 2);
+  if (norm_all) return launch_head_norm(o_raw, norm_w, gate, ld, gate_mode, 1, out, dtype, (long long)T, H * dv, eps, stream);
+  return launch_head_norm(o_raw, norm_w, gate, ld, gate_mode, H, out, dtype, (long long)T * H, dv, eps, stream);
+}

@@ -4,8 +4,10 @@
 ``S_t = decay_h S_{t-1} + k_t v_t^T`` and ``o_t = S_t^T q_t`` with one fixed ``decay_h`` per head and no other scale.
 The heads' ``o`` are concatenated and RMS-normed together (one weight per lane of the concatenation), multiplied by
 ``sigmoid(W_g x)`` and projected.  ``S`` starts at zero, is float32 and is carried per sequence as fixed-size state;
-the recurrence, the decays and the norm are float32 in every mode.  It runs on the scan of the gated linear
-attention, whose per-channel decays are here a constant vector."""
+the recurrence, the decays and the norm are float32 in every mode.  Steps of few tokens per sequence (decoding) run on
+the scan of the gated linear attention, whose per-channel decays are here a constant vector; prompts run chunk by
+chunk as float32 matrix products, which a constant decay allows (heads of up to 128 x 128 channels; larger ones take
+the scan there too)."""
 from __future__ import annotations
 
 import torch
@@ -16,6 +18,7 @@ from .base import Mixer, StateNeed, TensorSpec
 class LightningAttention(Mixer):
     """params: width, heads, dim, vdim, decay (one number in (0, 1] per head), eps.  names: q, k, v, g, norm, o."""
     graph_safe = True
+    CHUNKS_FROM = 8      # a step whose longest sequence brings at least this many tokens runs in chunks
 
     def tensor_specs(self):
         p, n = self.params, self.names
@@ -45,6 +48,10 @@ class LightningAttention(Mixer):
         self.w_in = rt.weight(torch.cat(ws, dim=0))
         self.w_o = rt.weight(tensors[n["o"]])
         self.norm_w = tensors[n["norm"]].float().contiguous()
+        self.in_chunks = rt.ops.lightning_chunks_supported(self.dk, self.dv)
+        if self.in_chunks:
+            rt.ops.lightning_chunks_init(rt.device)      # the kernels' shared memory, before any step is recorded
+            self.powers = rt.ops.decay_powers(decay, rt.device)
 
     def step_bytes(self, rows):
         return sum(w.w.numel() * w.w.element_size() for w in (self.w_in, self.w_o))
@@ -68,6 +75,9 @@ class LightningAttention(Mixer):
         T = proj.shape[0]
         o_raw = torch.zeros(T, self.H * self.dv, dtype=torch.float32, device=proj.device)
         out = torch.empty(T, self.H * self.dv, dtype=rt.dtype, device=proj.device)
+        if self.in_chunks and step.max_new >= self.CHUNKS_FROM and T > 4 * step.n_seqs:
+            return rt.ops.lightning_chunks(proj, self.powers, self.norm_w, self.eps, view.tensor, o_raw, out, step, self.H,
+                                           self.dk, self.dv, activation="silu", norm_all=True, gate="sigmoid")
         return rt.ops.gla_scan(proj, None, None, None, self.norm_w, self.eps, view.tensor, o_raw, out, step, self.H, self.dk,
                                self.dv, fixed_decay=self.decay, activation="silu", q_scale=1.0, norm_all=True, gate="sigmoid")
 

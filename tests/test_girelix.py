@@ -527,12 +527,17 @@ def test_keys_are_turned_in_adjacent_pairs_and_kept_unturned_as_values(dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
-@pytest.mark.parametrize("H,dk,dv", [(3, 12, 20), (10, 4, 250)], ids=["small", "norm_over_2500_lanes"])
-def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv):
-    """Three sequences in one step: a long prompt (walked in segments), a continuation from a state, one token from a
-    state; heads that forget at once, slowly and never; a state slot that is not in the step stays as it was.  The
-    recurrence is written out here once more, on rows that stand for the projections' results."""
+@pytest.mark.parametrize("H,dk,dv", [(3, 12, 20), (10, 4, 250), (2, 128, 128), (3, 70, 33)],
+                         ids=["small", "norm_over_2500_lanes", "largest_chunked_heads", "odd"])
+@pytest.mark.parametrize("form", ["scan", "chunks"])
+def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv, form):
+    """Three sequences in one step: a long prompt (walked in segments, or in chunks of 64 tokens whose last one is not
+    full), a continuation from a state, one token from a state; heads that forget at once, slowly and never; a state slot
+    that is not in the step stays as it was.  The recurrence is written out here once more, on rows that stand for the
+    projections' results."""
     from burn_lm_amd.csrc import ops
+    if form == "chunks" and not ops.lightning_chunks_supported(dk, dv):
+        pytest.skip("heads of this size are not run in chunks")
     dev = "cuda"
     r = dict(heads=H, dim=dk, vdim=dv, decay=([0.05, 0.999, 1.0] * 4)[:H])
     rng = np.random.default_rng(4)
@@ -562,9 +567,18 @@ def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv):
     state_dev = f32(states)
     T = sum(news)
     out = torch.empty(T, H * dv, dtype=dtype, device=dev)
-    ops.gla_scan(torch.from_numpy(proj).to(dev, dtype), None, None, None, f32(W["r.norm"]), 1e-5, state_dev,
-                 torch.zeros(T, H * dv, dtype=torch.float32, device=dev), out, step, H, dk, dv, segments=(3, 104),
-                 fixed_decay=f32(np.repeat(r["decay"], dk)), activation="silu", q_scale=1.0, norm_all=True, gate="sigmoid")
+    if form == "chunks":
+        ops.lightning_chunks_init(dev)
+        rows = torch.from_numpy(proj).to(dev, dtype)
+        before = rows.clone()
+        ops.lightning_chunks(rows, ops.decay_powers(r["decay"], dev), f32(W["r.norm"]), 1e-5, state_dev,
+                             torch.zeros(T, H * dv, dtype=torch.float32, device=dev), out, step, H, dk, dv,
+                             activation="silu", norm_all=True, gate="sigmoid")
+        assert torch.equal(rows, before)      # the activation happens on the way: the rows stay as they came
+    else:
+        ops.gla_scan(torch.from_numpy(proj).to(dev, dtype), None, None, None, f32(W["r.norm"]), 1e-5, state_dev,
+                     torch.zeros(T, H * dv, dtype=torch.float32, device=dev), out, step, H, dk, dv, segments=(3, 104),
+                     fixed_decay=f32(np.repeat(r["decay"], dk)), activation="silu", q_scale=1.0, norm_all=True, gate="sigmoid")
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     at = 0
     for (o, S), n, slot in zip(want, news, slots):
