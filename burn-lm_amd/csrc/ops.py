@@ -1337,9 +1337,10 @@ def decay_powers(decays, device):
 def lightning_chunks(proj, powers, norm_w, eps, state, o_raw, out, step, H, dk, dv, activation=None, norm_all=False,
                      gate="sigmoid"):
     """Linear attention with one constant decay per head over the prompts of a step, in chunks of 64 tokens as float32
-    matrix products: proj [T, >= 2 H dk + 2 H dv] (queries, keys, values, output-gate logits; not changed), powers as
+    matrix products: proj [T, >= 2 H dk + 2 H dv] (queries, keys, values, output-gate logits), powers as
     decay_powers gives them, state float32 [slots, H, dk, dv] read and left updated, o_raw float32 [T, H * dv], out
-    [T, H * dv] in proj's dtype.  activation, norm_all, gate as for gla_scan; the queries have no factor."""
+    [T, H * dv] in proj's dtype.  activation ("silu": proj's queries, keys and values are activated in place), norm_all,
+    gate as for gla_scan; the queries have no factor."""
     _gpu(proj, powers, norm_w, state, o_raw, out)
     T = proj.shape[0]
     _f32("o_raw", o_raw, T * H * dv); _f32("norm_w", norm_w, H * dv if norm_all else dv); _f32("state", state)

@@ -944,12 +944,12 @@ extern "C" int blm_gla_scan(void* proj, int dtype, int ld, const void* decay_in,
 //   O = (Q K^T * L) V + diag(a^(i+1)) Q S0,   L_ij = a^(i-j) for j <= i, else 0
 //   S_end = a^n S0 + (diag(a^(n-1-j)) K)^T V
 // All powers are at most one and come from a table pw [H][65] = a^0 .. a^64 (made in double precision), so no quotient or
-// running product of decays appears and a fast decay cannot overflow.  Three kernels: lc_state (every chunk's own
-// contribution (diag(..) K)^T V, the first chunk's with the sequence's state), gla_carry (the chunks' start states in
-// order, and the sequence's new state), lc_out (the chunk's results).  Operands are staged through shared memory in the
-// rows' type (the activated queries, keys and values are rounded to it, as a projection's output is) and multiplied by
-// 32x32x2 float32 matrix instructions: lane l holds row l % 32 of the left operand and column l % 32 of the right one at
-// depth l / 32; result register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
+// running product of decays appears and a fast decay cannot overflow.  Kernels: silu_rows (the activation, once, in
+// place), lc_state (every chunk's own contribution (diag(..) K)^T V, the first chunk's with the sequence's state),
+// gla_carry (the chunks' start states in order, and the sequence's new state), lc_out (the chunk's results).  Operands
+// are staged through shared memory in the rows' type, 16 bytes per lane and load, and multiplied by 32x32x2 float32
+// matrix instructions: lane l holds row l % 32 of the left operand and column l % 32 of the right one at depth l / 32;
+// result register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
 // Heads of up to 128 key and 128 value channels, padded to multiples of 32 with zeros.
 // ---------------------------------------------------------------------------------------
 #define LC_CHUNK 64
@@ -962,16 +962,77 @@ typedef float lc_acc __attribute__((ext_vector_type(16)));
 template <typename TA>
 __device__ __forceinline__ int lc_row_pad() { return sizeof(TA) == 4 ? 1 : 2; }      // an odd number of 4-byte words per row
 
+// SiLU rounded to the rows' type.  Rows of 16 bits take the hardware's exponential and reciprocal, whose errors (about
+// 1e-6 of the result) are far below that rounding; float rows take the exact functions.
 template <typename TA>
-__device__ __forceinline__ float lc_read(const TA* __restrict__ p, int act) {
-  const float x = to_float(*p);
-  return act ? to_float(from_float<TA>(blm_silu(x))) : x;
+__device__ __forceinline__ TA lc_silu(TA v) {
+  const float x = to_float(v);
+  if (sizeof(TA) == 4) return from_float<TA>(blm_silu(x));
+  return from_float<TA>(x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * x)));
+}
+
+// SiLU in place on the first `cols` columns of every row, 16 bytes per lane (cols and ld multiples of that many elements,
+// rows aligned to 16 bytes).
+template <typename TA>
+__global__ void silu_rows_wide_kernel(TA* __restrict__ proj, int ld, int cols, long long n_vec) {
+  constexpr int VEC = 16 / sizeof(TA);
+  const int per_row = cols / VEC;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n_vec; e += stride) {
+    const long long t = e / per_row;
+    uint4* at = reinterpret_cast<uint4*>(proj + (size_t)t * ld + (size_t)(e - t * per_row) * VEC);
+    uint4 raw = *at;
+    TA* vals = reinterpret_cast<TA*>(&raw);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) vals[k] = lc_silu(vals[k]);
+    *at = raw;
+  }
+}
+
+// A chunk's rows of one head, `width` channels from column col0 on, into shared memory dst [64][row_ld] as they are: the
+// tokens from n on and the channels from width up to the padded width WP arrive as zeros.  Where rows and width allow,
+// every lane takes 16 bytes at a time, has four such loads under way before it turns to the first, and leaves them as
+// four 4-byte words (row_ld and the 16-byte pieces keep every word aligned).
+template <typename TA>
+__device__ __forceinline__ void lc_stage(const TA* __restrict__ rows, int ld, int col0, int width, int WP, int n,
+                                         TA* __restrict__ dst, int row_ld) {
+  constexpr int VEC = 16 / sizeof(TA);
+  const TA* src = rows + col0;
+  if (width % VEC == 0 && ld % VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+    const int per_row = width / VEC, items = LC_CHUNK * per_row;
+    for (int base = threadIdx.x; base < items; base += 4 * LC_THREADS) {
+      uint4 raw[4];
+      int at[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int e = base + u * LC_THREADS, j = e / per_row, i = (e - j * per_row) * VEC;
+        at[u] = e < items ? j * row_ld + i : -1;
+        raw[u] = (e < items && j < n) ? *reinterpret_cast<const uint4*>(src + (size_t)j * ld + i) : uint4{0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (at[u] >= 0) {
+          uint32_t* w = reinterpret_cast<uint32_t*>(dst + at[u]);
+          w[0] = raw[u].x; w[1] = raw[u].y; w[2] = raw[u].z; w[3] = raw[u].w;
+        }
+      }
+    }
+    if (WP > width) {
+      const int extra = WP - width;
+      for (int e = threadIdx.x; e < LC_CHUNK * extra; e += LC_THREADS) dst[(e / extra) * row_ld + width + e % extra] = from_float<TA>(0.f);
+    }
+  } else {
+    for (int e = threadIdx.x; e < LC_CHUNK * WP; e += LC_THREADS) {
+      const int j = e / WP, i = e - j * WP;
+      dst[j * row_ld + i] = (j < n && i < width) ? src[(size_t)j * ld + i] : from_float<TA>(0.f);
+    }
+  }
 }
 
 // seg_end [B][n_seg][H][dk][dv], seg_start likewise (only chunk 0 is written here), seg_decay [B][n_seg][H][dk]
 template <typename TA>
 __global__ void __launch_bounds__(LC_THREADS)
-    lc_state_kernel(const TA* __restrict__ proj, int ld, int act, const float* __restrict__ pw, const float* __restrict__ state,
+    lc_state_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ pw, const float* __restrict__ state,
                     float* __restrict__ seg_end, float* __restrict__ seg_start, float* __restrict__ seg_decay,
                     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk, int dv, int n_seg) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lc_sm[];
@@ -981,18 +1042,14 @@ __global__ void __launch_bounds__(LC_THREADS)
   if (slot < 0 || t0 >= n_new) return;
   const int n = min(LC_CHUNK, n_new - t0);
   const int DKP = (dk + 31) & ~31, DVP = (dv + 31) & ~31;
-  float* Kf = reinterpret_cast<float*>(lc_sm);                      // [64][DKP], each key times a^(n-1-j)
-  TA* Vs = reinterpret_cast<TA*>(Kf + LC_CHUNK * DKP);              // [64][DVP]
+  float* wj = reinterpret_cast<float*>(lc_sm);                      // [64]: a^(n-1-j), zero from n on
+  TA* Ks = reinterpret_cast<TA*>(wj + LC_CHUNK);                    // [64][DKP]
+  TA* Vs = Ks + LC_CHUNK * DKP;                                     // [64][DVP]
   const float* pwh = pw + h * (LC_CHUNK + 1);
   const TA* rows = proj + (size_t)(first + t0) * ld;
-  for (int e = threadIdx.x; e < LC_CHUNK * DKP; e += LC_THREADS) {
-    const int j = e / DKP, i = e - j * DKP;
-    Kf[e] = (j < n && i < dk) ? lc_read(rows + (size_t)j * ld + (size_t)H * dk + h * dk + i, act) * pwh[n - 1 - j] : 0.f;
-  }
-  for (int e = threadIdx.x; e < LC_CHUNK * DVP; e += LC_THREADS) {
-    const int j = e / DVP, i = e - j * DVP;
-    Vs[e] = from_float<TA>((j < n && i < dv) ? lc_read(rows + (size_t)j * ld + (size_t)2 * H * dk + h * dv + i, act) : 0.f);
-  }
+  lc_stage<TA>(rows, ld, H * dk + h * dk, dk, DKP, n, Ks, DKP);
+  lc_stage<TA>(rows, ld, 2 * H * dk + h * dv, dv, DVP, n, Vs, DVP);
+  if (threadIdx.x < LC_CHUNK) wj[threadIdx.x] = threadIdx.x < n ? pwh[n - 1 - threadIdx.x] : 0.f;
   __syncthreads();
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int lr = lane & 31, lk = lane >> 5;
@@ -1003,39 +1060,49 @@ __global__ void __launch_bounds__(LC_THREADS)
   for (int s = 0; s < 4; ++s)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[s][r] = 0.f;
-  for (int k0 = 0; k0 < depth; k0 += 2) {
-    const float* krow = Kf + (k0 + lk) * DKP + lr;
-    const TA* vrow = Vs + (k0 + lk) * DVP + lr;
+  int k_at[4], v_at[4];      // where the wavefront's tiles start in a row of keys and of values
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int t = wave + 4 * s;
-      if (t < tiles) {
-        const int tr = t / NV, tc = t - tr * NV;
-        acc[s] = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[tr * 32], to_float(vrow[tc * 32]), acc[s], 0, 0, 0);
-      }
-    }
+  for (int s = 0; s < 4; ++s) {
+    const int t = min(wave + 4 * s, tiles - 1), tr = t / NV;
+    k_at[s] = tr * 32 + lr;
+    v_at[s] = (t - tr * NV) * 32 + lr;
+  }
+  // The weight of token j goes onto its values.  Every wavefront multiplies four tiles whether it has that many or not (a
+  // wavefront with fewer repeats its last one into accumulators that are never stored): a matrix instruction under a
+  // condition would make the compiler move its sixteen result registers about in every turn of the loop.
+#pragma unroll 4
+  for (int k0 = 0; k0 < depth; k0 += 2) {
+    const TA* krow = Ks + (k0 + lk) * DKP;
+    const TA* vrow = Vs + (k0 + lk) * DVP;
+    const float w = wj[k0 + lk];
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      acc[s] = __builtin_amdgcn_mfma_f32_32x32x2f32(to_float(krow[k_at[s]]), to_float(vrow[v_at[s]]) * w, acc[s], 0, 0, 0);
   }
   const size_t per = (size_t)dk * dv;
   const size_t at = (((size_t)b * n_seg + c) * H + h) * per;
   const float* S_old = state + ((size_t)slot * H + h) * per;
   const float fade = pwh[n];
+  const bool whole = (dk & 31) == 0 && (dv & 31) == 0;
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
     const int t = wave + 4 * s;
     if (t < tiles) {
       const int tr = t / NV, tc = t - tr * NV;
-      const int col = tc * 32 + lr;
+      const int col = tc * 32 + lr, i0 = tr * 32 + 4 * lk;
+      const size_t o = (size_t)i0 * dv + col;
+      float* end_p = seg_end + at + o;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int i = tr * 32 + 8 * (r / 4) + 4 * lk + (r & 3);
-        if (i < dk && col < dv) {
+        const int di = 8 * (r / 4) + (r & 3);
+        if (whole || (i0 + di < dk && col < dv)) {
           float v = acc[s][r];
           if (c == 0) {
-            const float old = S_old[(size_t)i * dv + col];
-            seg_start[at + (size_t)i * dv + col] = old;
+            const float old = S_old[o + (size_t)di * dv];
+            seg_start[at + o + (size_t)di * dv] = old;
             v = fmaf(fade, old, v);
           }
-          seg_end[at + (size_t)i * dv + col] = v;
+          end_p[(size_t)di * dv] = v;
         }
       }
     }
@@ -1045,7 +1112,7 @@ __global__ void __launch_bounds__(LC_THREADS)
 
 template <typename TA>
 __global__ void __launch_bounds__(LC_THREADS)
-    lc_out_kernel(const TA* __restrict__ proj, int ld, int act, const float* __restrict__ pw, const float* __restrict__ seg_start,
+    lc_out_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ pw, const float* __restrict__ seg_start,
                   float* __restrict__ o_raw, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk,
                   int dv, int n_seg) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lc_sm[];
@@ -1062,16 +1129,9 @@ __global__ void __launch_bounds__(LC_THREADS)
   TA* Ks = Qs + LC_CHUNK * SK;                                      // [64][SK]
   TA* Vs = Ks + LC_CHUNK * SK;                                      // [64][DVP]
   const TA* rows = proj + (size_t)(first + t0) * ld;
-  for (int e = threadIdx.x; e < LC_CHUNK * DKP; e += LC_THREADS) {
-    const int j = e / DKP, i = e - j * DKP;
-    const bool in = j < n && i < dk;
-    Qs[j * SK + i] = from_float<TA>(in ? lc_read(rows + (size_t)j * ld + h * dk + i, act) : 0.f);
-    Ks[j * SK + i] = from_float<TA>(in ? lc_read(rows + (size_t)j * ld + (size_t)H * dk + h * dk + i, act) : 0.f);
-  }
-  for (int e = threadIdx.x; e < LC_CHUNK * DVP; e += LC_THREADS) {
-    const int j = e / DVP, i = e - j * DVP;
-    Vs[e] = from_float<TA>((j < n && i < dv) ? lc_read(rows + (size_t)j * ld + (size_t)2 * H * dk + h * dv + i, act) : 0.f);
-  }
+  lc_stage<TA>(rows, ld, h * dk, dk, DKP, n, Qs, SK);
+  lc_stage<TA>(rows, ld, H * dk + h * dk, dk, DKP, n, Ks, SK);
+  lc_stage<TA>(rows, ld, 2 * H * dk + h * dv, dv, DVP, n, Vs, DVP);
   if (threadIdx.x <= LC_CHUNK) pws[threadIdx.x] = pw[h * (LC_CHUNK + 1) + threadIdx.x];
   __syncthreads();
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
@@ -1085,7 +1145,7 @@ __global__ void __launch_bounds__(LC_THREADS)
     for (int r = 0; r < 16; ++r) sc[r] = 0.f;
     const TA* qrow = Qs + (ti * 32 + lr) * SK + lk;
     const TA* krow = Ks + (tj * 32 + lr) * SK + lk;
-#pragma unroll 4
+#pragma unroll 8
     for (int k0 = 0; k0 < depth_k; k0 += 2)
       sc = __builtin_amdgcn_mfma_f32_32x32x2f32(to_float(qrow[k0]), to_float(krow[k0]), sc, 0, 0, 0);
     const int j = tj * 32 + lr;
@@ -1098,25 +1158,28 @@ __global__ void __launch_bounds__(LC_THREADS)
   __syncthreads();
   const int NV = DVP / 32;
   const int ti = wave & 1, tc0 = wave >> 1;
+  const bool two = tc0 + 2 < NV;
+  // A wavefront without a first or second tile of its own repeats the head's last column tile and stores nothing of it:
+  // no matrix instruction stands under a condition (see lc_state_kernel).
+  const int ca = min(tc0, NV - 1) * 32 + lr, cb = min(tc0 + 2, NV - 1) * 32 + lr;
   lc_acc acc[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[s][r] = 0.f;
-  // what the chunk's start state gives: Q S0, row i times a^(i+1)
+  // what the chunk's start state gives: Q S0, row i times a^(i+1).  Columns from dv on and the row behind an odd dk are
+  // read from the last valid column and row: such columns are never stored, and that row meets zeros of Q.
   {
     const float* S0 = seg_start + (((size_t)b * n_seg + c) * H + h) * (size_t)dk * dv;
     const TA* qrow = Qs + (ti * 32 + lr) * SK + lk;
-    const int col0 = tc0 * 32 + lr, col1 = (tc0 + 2) * 32 + lr;
-    const bool in0 = tc0 < NV && col0 < dv, in1 = tc0 + 2 < NV && col1 < dv;
-#pragma unroll 4
+    const float* s0 = S0 + min(ca, dv - 1);
+    const float* s1 = S0 + min(cb, dv - 1);
+#pragma unroll 8
     for (int k0 = 0; k0 < depth_k; k0 += 2) {
-      const int kk = k0 + lk;
+      const size_t row = (size_t)min(k0 + lk, dk - 1) * dv;
       const float a = to_float(qrow[k0]);
-      const float s0 = (in0 && kk < dk) ? S0[(size_t)kk * dv + col0] : 0.f;
-      const float s1 = (in1 && kk < dk) ? S0[(size_t)kk * dv + col1] : 0.f;
-      if (tc0 < NV) acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s0, acc[0], 0, 0, 0);
-      if (tc0 + 2 < NV) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s1, acc[1], 0, 0, 0);
+      acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s0[row], acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s1[row], acc[1], 0, 0, 0);
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -1128,24 +1191,26 @@ __global__ void __launch_bounds__(LC_THREADS)
   // what the chunk's own tokens give: (scores * L) V, over the keys up to the row tile's last row
   {
     const float* arow = As + (ti * 32 + lr) * LC_A_LD + lk;
-    const TA* vrow = Vs + lk * DVP + lr;
+    const TA* v0 = Vs + lk * DVP + ca;
+    const TA* v1 = Vs + lk * DVP + cb;
     const int depth = min((ti + 1) * 32, (n + 1) & ~1);
-#pragma unroll 4
+#pragma unroll 8
     for (int k0 = 0; k0 < depth; k0 += 2) {
       const float a = arow[k0];
-      if (tc0 < NV) acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(vrow[k0 * DVP + tc0 * 32]), acc[0], 0, 0, 0);
-      if (tc0 + 2 < NV) acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(vrow[k0 * DVP + (tc0 + 2) * 32]), acc[1], 0, 0, 0);
+      acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(v0[k0 * DVP]), acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(v1[k0 * DVP]), acc[1], 0, 0, 0);
     }
   }
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
-    const int tc = tc0 + 2 * s;
-    const int col = tc * 32 + lr;
-    if (tc < NV && col < dv) {
+    const int col = (tc0 + 2 * s) * 32 + lr;
+    if ((s == 0 ? tc0 < NV : two) && col < dv) {
+      const int i0 = ti * 32 + 4 * lk;
+      float* o = o_raw + ((size_t)(first + t0 + i0) * H + h) * dv + col;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int i = ti * 32 + 8 * (r / 4) + 4 * lk + (r & 3);
-        if (i < n) o_raw[((size_t)(first + t0 + i) * H + h) * dv + col] = acc[s][r];
+        const int di = 8 * (r / 4) + (r & 3);
+        if (i0 + di < n) o[(size_t)di * H * dv] = acc[s][r];
       }
     }
   }
@@ -1153,7 +1218,7 @@ __global__ void __launch_bounds__(LC_THREADS)
 
 static size_t lc_state_lds(int dk, int dv, int dtype) {
   const int DKP = (dk + 31) & ~31, DVP = (dv + 31) & ~31;
-  return (size_t)LC_CHUNK * DKP * sizeof(float) + (size_t)LC_CHUNK * DVP * (dtype == BLM_F32 ? 4 : 2);
+  return (size_t)LC_CHUNK * sizeof(float) + (size_t)LC_CHUNK * (DKP + DVP) * (dtype == BLM_F32 ? 4 : 2);
 }
 static size_t lc_out_lds(int dk, int dv, int dtype) {
   const int DKP = (dk + 31) & ~31, DVP = (dv + 31) & ~31;
@@ -1183,8 +1248,8 @@ extern "C" int blm_lightning_chunks_supported(int dk, int dv) { return (dk >= 1 
 // proj as for blm_gla_scan (queries, keys, values, output-gate logits); pw [H][65] float: powers 0 .. 64 of every head's
 // decay; n_seg: chunks of 64 tokens that cover the longest sequence of the step; seg_end, seg_start [B][n_seg][H][dk][dv],
 // seg_decay [B][n_seg][H][dk] float.  state is read and left updated; o_raw [T][H*dv] float; out [T][H*dv] in proj's type.
-// act_mode, norm_all, gate_mode as for blm_gla_scan (the activation happens on the way into shared memory: proj is not changed).
-extern "C" int blm_lightning_chunks(const void* proj, int dtype, int ld, const float* pw, const float* norm_w, float eps,
+// act_mode, norm_all, gate_mode as for blm_gla_scan (act_mode 1 activates proj's queries, keys and values in place).
+extern "C" int blm_lightning_chunks(void* proj, int dtype, int ld, const float* pw, const float* norm_w, float eps,
                                     float* state, float* o_raw, void* out, const int* cu_seqlens, const int* seq_slots, int T,
                                     int B, int H, int dk, int dv, int max_new, int n_seg, float* seg_end, float* seg_start,
                                     float* seg_decay, int act_mode, int norm_all, int gate_mode, hipStream_t stream) {
@@ -1200,12 +1265,27 @@ extern "C" int blm_lightning_chunks(const void* proj, int dtype, int ld, const f
               "lightning_chunks: blm_lightning_chunks_init has not run on device %d", dev);
   const size_t lds_a = lc_state_lds(dk, dv, dtype), lds_c = lc_out_lds(dk, dv, dtype);
   BLM_REQUIRE(lds_a <= LC_LDS_LIMIT && lds_c <= LC_LDS_LIMIT, "lightning_chunks: %zu bytes of shared memory are too many", lds_c);
+  if (act_mode == 1) {
+    const int cols = 2 * H * dk + H * dv, vec = dtype == BLM_F32 ? 4 : 8;
+    if (cols % vec == 0 && ld % vec == 0 && ((uintptr_t)proj & 15) == 0) {
+      const long long n = (long long)T * (cols / vec);
+      const unsigned ablocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+      if (dtype == BLM_F32) hipLaunchKernelGGL(silu_rows_wide_kernel<float>, dim3(ablocks), dim3(256), 0, stream, (float*)proj, ld, cols, n);
+      else hipLaunchKernelGGL(silu_rows_wide_kernel<bf16>, dim3(ablocks), dim3(256), 0, stream, (bf16*)proj, ld, cols, n);
+    } else {
+      const long long n = (long long)T * cols;
+      const unsigned ablocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+      if (dtype == BLM_F32) hipLaunchKernelGGL(silu_rows_kernel<float>, dim3(ablocks), dim3(256), 0, stream, (float*)proj, ld, cols, n);
+      else hipLaunchKernelGGL(silu_rows_kernel<bf16>, dim3(ablocks), dim3(256), 0, stream, (bf16*)proj, ld, cols, n);
+    }
+    BLM_LAUNCH_CHECK("silu_rows");
+  }
   const dim3 grid((unsigned)n_seg, (unsigned)H, (unsigned)B);
   if (dtype == BLM_F32)
-    hipLaunchKernelGGL(lc_state_kernel<float>, grid, dim3(LC_THREADS), lds_a, stream, (const float*)proj, ld, act_mode, pw, state,
+    hipLaunchKernelGGL(lc_state_kernel<float>, grid, dim3(LC_THREADS), lds_a, stream, (const float*)proj, ld, pw, state,
                        seg_end, seg_start, seg_decay, cu_seqlens, seq_slots, H, dk, dv, n_seg);
   else
-    hipLaunchKernelGGL(lc_state_kernel<bf16>, grid, dim3(LC_THREADS), lds_a, stream, (const bf16*)proj, ld, act_mode, pw, state,
+    hipLaunchKernelGGL(lc_state_kernel<bf16>, grid, dim3(LC_THREADS), lds_a, stream, (const bf16*)proj, ld, pw, state,
                        seg_end, seg_start, seg_decay, cu_seqlens, seq_slots, H, dk, dv, n_seg);
   BLM_LAUNCH_CHECK("lc_state");
   const size_t per = (size_t)H * dk * dv;
@@ -1214,10 +1294,10 @@ extern "C" int blm_lightning_chunks(const void* proj, int dtype, int ld, const f
                      seq_slots, H, dk, dv, n_seg, LC_CHUNK);
   BLM_LAUNCH_CHECK("gla_carry");
   if (dtype == BLM_F32)
-    hipLaunchKernelGGL(lc_out_kernel<float>, grid, dim3(LC_THREADS), lds_c, stream, (const float*)proj, ld, act_mode, pw, seg_start,
+    hipLaunchKernelGGL(lc_out_kernel<float>, grid, dim3(LC_THREADS), lds_c, stream, (const float*)proj, ld, pw, seg_start,
                        o_raw, cu_seqlens, seq_slots, H, dk, dv, n_seg);
   else
-    hipLaunchKernelGGL(lc_out_kernel<bf16>, grid, dim3(LC_THREADS), lds_c, stream, (const bf16*)proj, ld, act_mode, pw, seg_start,
+    hipLaunchKernelGGL(lc_out_kernel<bf16>, grid, dim3(LC_THREADS), lds_c, stream, (const bf16*)proj, ld, pw, seg_start,
                        o_raw, cu_seqlens, seq_slots, H, dk, dv, n_seg);
   BLM_LAUNCH_CHECK("lc_out");
   const char* gate = (const char*)proj + (size_t)(2 * H * dk + H * dv) * (dtype == BLM_F32 ? 4 : 2);

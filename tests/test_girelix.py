@@ -569,12 +569,9 @@ def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv, form):
     out = torch.empty(T, H * dv, dtype=dtype, device=dev)
     if form == "chunks":
         ops.lightning_chunks_init(dev)
-        rows = torch.from_numpy(proj).to(dev, dtype)
-        before = rows.clone()
-        ops.lightning_chunks(rows, ops.decay_powers(r["decay"], dev), f32(W["r.norm"]), 1e-5, state_dev,
+        ops.lightning_chunks(torch.from_numpy(proj).to(dev, dtype), ops.decay_powers(r["decay"], dev), f32(W["r.norm"]), 1e-5, state_dev,
                              torch.zeros(T, H * dv, dtype=torch.float32, device=dev), out, step, H, dk, dv,
                              activation="silu", norm_all=True, gate="sigmoid")
-        assert torch.equal(rows, before)      # the activation happens on the way: the rows stay as they came
     else:
         ops.gla_scan(torch.from_numpy(proj).to(dev, dtype), None, None, None, f32(W["r.norm"]), 1e-5, state_dev,
                      torch.zeros(T, H * dv, dtype=torch.float32, device=dev), out, step, H, dk, dv, segments=(3, 104),
