@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 36
+ABI_VERSION = 37
 _lib = None
 _lock = threading.Lock()
 
@@ -41,7 +41,7 @@ _SIGNATURES = {
     "blm_lightning_chunks_init": [],
     "blm_lightning_chunks_supported": [_c_int, _c_int],
     "blm_lightning_chunks": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                             _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                             _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p,
                              _c_int, _c_int, _c_int, _c_void_p],
     "blm_qkv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -1353,10 +1353,9 @@ def lightning_chunks(proj, powers, norm_w, eps, state, o_raw, out, step, H, dk, 
     B, n_seg = step.n_seqs, -(-step.max_new // LIGHTNING_CHUNK)
     seg_end = torch.empty(B, n_seg, H, dk, dv, dtype=torch.float32, device=proj.device)
     seg_start = torch.empty_like(seg_end)
-    seg_decay = torch.empty(B, n_seg, H, dk, dtype=torch.float32, device=proj.device)
     _call("blm_lightning_chunks", proj.data_ptr(), _code(proj), proj.stride(0), powers.data_ptr(), norm_w.data_ptr(), float(eps),
           state.data_ptr(), o_raw.data_ptr(), out.data_ptr(), step.cu_seqlens.data_ptr(), step.seq_slots.data_ptr(), T, B, H, dk,
-          dv, step.max_new, n_seg, seg_end.data_ptr(), seg_start.data_ptr(), seg_decay.data_ptr(),
+          dv, step.max_new, n_seg, seg_end.data_ptr(), seg_start.data_ptr(),
           1 if activation == "silu" else 0, 1 if norm_all else 0, GATE_MODES[gate], _stream())
     return out
 

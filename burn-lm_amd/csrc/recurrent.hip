@@ -945,8 +945,8 @@ extern "C" int blm_gla_scan(void* proj, int dtype, int ld, const void* decay_in,
 //   S_end = a^n S0 + (diag(a^(n-1-j)) K)^T V
 // All powers are at most one and come from a table pw [H][65] = a^0 .. a^64 (made in double precision), so no quotient or
 // running product of decays appears and a fast decay cannot overflow.  Kernels: silu_rows (the activation, once, in
-// place), lc_state (every chunk's own contribution (diag(..) K)^T V, the first chunk's with the sequence's state),
-// gla_carry (the chunks' start states in order, and the sequence's new state), lc_out (the chunk's results).  Operands
+// place), lc_state (every chunk's own contribution (diag(..) K)^T V), lc_carry (the chunks' start states in order, from
+// the sequence's state, and its new state), lc_out (the chunk's results).  Operands
 // are staged through shared memory in the rows' type, 16 bytes per lane and load, and multiplied by 32x32x2 float32
 // matrix instructions: lane l holds row l % 32 of the left operand and column l % 32 of the right one at depth l / 32;
 // result register r of lane l is row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32.
@@ -956,6 +956,7 @@ extern "C" int blm_gla_scan(void* proj, int dtype, int ld, const void* decay_in,
 #define LC_MAX 128
 #define LC_THREADS 256
 #define LC_A_LD (LC_CHUNK + 1)
+#define LC_STEPS 8      // matrix instructions written out per turn of a loop over depth: 16 steps of depth
 #define LC_LDS_LIMIT (128 * 1024)
 typedef float lc_acc __attribute__((ext_vector_type(16)));
 
@@ -989,51 +990,70 @@ __global__ void silu_rows_wide_kernel(TA* __restrict__ proj, int ld, int cols, l
   }
 }
 
-// A chunk's rows of one head, `width` channels from column col0 on, into shared memory dst [64][row_ld] as they are: the
-// tokens from n on and the channels from width up to the padded width WP arrive as zeros.  Where rows and width allow,
-// every lane takes 16 bytes at a time, has four such loads under way before it turns to the first, and leaves them as
-// four 4-byte words (row_ld and the 16-byte pieces keep every word aligned).
-template <typename TA>
-__device__ __forceinline__ void lc_stage(const TA* __restrict__ rows, int ld, int col0, int width, int WP, int n,
-                                         TA* __restrict__ dst, int row_ld) {
+// A chunk's rows of one head into shared memory as they are, for N operands at once (queries, keys, values): operand p
+// is `width[p]` channels from column col0[p] on and arrives in dst[p] [64][row_ld[p]]; the tokens from n on and the channels
+// from width up to the padded width WP arrive as zeros.  Where rows and widths allow, every lane takes 16 bytes at a
+// time, has all its loads of all operands under way before it turns to the first (one trip to memory, not one per
+// operand), and leaves them as 4-byte words (row_ld and the 16-byte pieces keep every word aligned).
+template <typename TA, int N>
+struct LcOperands {
+  int col0[N], width[N], WP[N], row_ld[N];
+  TA* dst[N];
+};
+
+template <typename TA, int N>
+__device__ __forceinline__ void lc_stage(const TA* __restrict__ rows, int ld, int n, const LcOperands<TA, N>& op) {
   constexpr int VEC = 16 / sizeof(TA);
-  const TA* src = rows + col0;
-  if (width % VEC == 0 && ld % VEC == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
-    const int per_row = width / VEC, items = LC_CHUNK * per_row;
-    for (int base = threadIdx.x; base < items; base += 4 * LC_THREADS) {
-      uint4 raw[4];
-      int at[4];
+  bool wide = ld % VEC == 0 && (reinterpret_cast<uintptr_t>(rows) & 15) == 0;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int e = base + u * LC_THREADS, j = e / per_row, i = (e - j * per_row) * VEC;
-        at[u] = e < items ? j * row_ld + i : -1;
-        raw[u] = (e < items && j < n) ? *reinterpret_cast<const uint4*>(src + (size_t)j * ld + i) : uint4{0u, 0u, 0u, 0u};
+  for (int p = 0; p < N; ++p) wide = wide && op.width[p] % VEC == 0 && op.col0[p] % VEC == 0 && op.width[p] <= LC_MAX;
+  if (wide) {
+    // up to 64 * 128 / VEC pieces per operand: at most 4 (16-bit rows) or 8 (float rows) per lane
+    constexpr int PER = (LC_CHUNK * LC_MAX / VEC + LC_THREADS - 1) / LC_THREADS;
+    uint4 raw[N][PER];
+    int at[N][PER];
+#pragma unroll
+    for (int p = 0; p < N; ++p) {
+      const int per_row = op.width[p] / VEC, items = LC_CHUNK * per_row;
+      const TA* src = rows + op.col0[p];
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int e = threadIdx.x + u * LC_THREADS, j = e / per_row, i = (e - j * per_row) * VEC;
+        at[p][u] = e < items ? j * op.row_ld[p] + i : -1;
+        raw[p][u] = (e < items && j < n) ? *reinterpret_cast<const uint4*>(src + (size_t)j * ld + i) : uint4{0u, 0u, 0u, 0u};
       }
+    }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (at[u] >= 0) {
-          uint32_t* w = reinterpret_cast<uint32_t*>(dst + at[u]);
-          w[0] = raw[u].x; w[1] = raw[u].y; w[2] = raw[u].z; w[3] = raw[u].w;
+    for (int p = 0; p < N; ++p) {
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        if (at[p][u] >= 0) {
+          uint32_t* w = reinterpret_cast<uint32_t*>(op.dst[p] + at[p][u]);
+          w[0] = raw[p][u].x; w[1] = raw[p][u].y; w[2] = raw[p][u].z; w[3] = raw[p][u].w;
         }
       }
-    }
-    if (WP > width) {
-      const int extra = WP - width;
-      for (int e = threadIdx.x; e < LC_CHUNK * extra; e += LC_THREADS) dst[(e / extra) * row_ld + width + e % extra] = from_float<TA>(0.f);
+      if (op.WP[p] > op.width[p]) {
+        const int extra = op.WP[p] - op.width[p];
+        for (int e = threadIdx.x; e < LC_CHUNK * extra; e += LC_THREADS)
+          op.dst[p][(e / extra) * op.row_ld[p] + op.width[p] + e % extra] = from_float<TA>(0.f);
+      }
     }
   } else {
-    for (int e = threadIdx.x; e < LC_CHUNK * WP; e += LC_THREADS) {
-      const int j = e / WP, i = e - j * WP;
-      dst[j * row_ld + i] = (j < n && i < width) ? src[(size_t)j * ld + i] : from_float<TA>(0.f);
+#pragma unroll
+    for (int p = 0; p < N; ++p) {
+      const TA* src = rows + op.col0[p];
+      for (int e = threadIdx.x; e < LC_CHUNK * op.WP[p]; e += LC_THREADS) {
+        const int j = e / op.WP[p], i = e - j * op.WP[p];
+        op.dst[p][j * op.row_ld[p] + i] = (j < n && i < op.width[p]) ? src[(size_t)j * ld + i] : from_float<TA>(0.f);
+      }
     }
   }
 }
 
-// seg_end [B][n_seg][H][dk][dv], seg_start likewise (only chunk 0 is written here), seg_decay [B][n_seg][H][dk]
+// seg_end [B][n_seg][H][dk][dv]: what the chunk's own tokens add to the state by the chunk's end
 template <typename TA>
 __global__ void __launch_bounds__(LC_THREADS)
-    lc_state_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ pw, const float* __restrict__ state,
-                    float* __restrict__ seg_end, float* __restrict__ seg_start, float* __restrict__ seg_decay,
+    lc_state_kernel(const TA* __restrict__ proj, int ld, const float* __restrict__ pw, float* __restrict__ seg_end,
                     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots, int H, int dk, int dv, int n_seg) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lc_sm[];
   const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -1047,14 +1067,18 @@ __global__ void __launch_bounds__(LC_THREADS)
   TA* Vs = Ks + LC_CHUNK * DKP;                                     // [64][DVP]
   const float* pwh = pw + h * (LC_CHUNK + 1);
   const TA* rows = proj + (size_t)(first + t0) * ld;
-  lc_stage<TA>(rows, ld, H * dk + h * dk, dk, DKP, n, Ks, DKP);
-  lc_stage<TA>(rows, ld, 2 * H * dk + h * dv, dv, DVP, n, Vs, DVP);
+  {
+    LcOperands<TA, 2> op;
+    op.col0[0] = H * dk + h * dk; op.width[0] = dk; op.WP[0] = DKP; op.row_ld[0] = DKP; op.dst[0] = Ks;
+    op.col0[1] = 2 * H * dk + h * dv; op.width[1] = dv; op.WP[1] = DVP; op.row_ld[1] = DVP; op.dst[1] = Vs;
+    lc_stage<TA, 2>(rows, ld, n, op);
+  }
   if (threadIdx.x < LC_CHUNK) wj[threadIdx.x] = threadIdx.x < n ? pwh[n - 1 - threadIdx.x] : 0.f;
   __syncthreads();
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int lr = lane & 31, lk = lane >> 5;
   const int NV = DVP / 32, tiles = (DKP / 32) * NV;
-  const int depth = (n + 1) & ~1;
+  const int depth = (n + 2 * LC_STEPS - 1) & ~(2 * LC_STEPS - 1);
   lc_acc acc[4];
 #pragma unroll
   for (int s = 0; s < 4; ++s)
@@ -1070,19 +1094,21 @@ __global__ void __launch_bounds__(LC_THREADS)
   // The weight of token j goes onto its values.  Every wavefront multiplies four tiles whether it has that many or not (a
   // wavefront with fewer repeats its last one into accumulators that are never stored): a matrix instruction under a
   // condition would make the compiler move its sixteen result registers about in every turn of the loop.
-#pragma unroll 4
-  for (int k0 = 0; k0 < depth; k0 += 2) {
-    const TA* krow = Ks + (k0 + lk) * DKP;
-    const TA* vrow = Vs + (k0 + lk) * DVP;
-    const float w = wj[k0 + lk];
+  // (A loop whose turns are counted at run time is not unrolled around matrix instructions: sixteen steps of depth are
+  // written out per turn, and the depth is rounded up to that; what lies behind the chunk's tokens is zeros.)
+  for (int kb = 0; kb < depth; kb += 2 * LC_STEPS) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
-      acc[s] = __builtin_amdgcn_mfma_f32_32x32x2f32(to_float(krow[k_at[s]]), to_float(vrow[v_at[s]]) * w, acc[s], 0, 0, 0);
+    for (int u = 0; u < LC_STEPS; ++u) {
+      const int k0 = kb + 2 * u;
+      const TA* krow = Ks + (k0 + lk) * DKP;
+      const TA* vrow = Vs + (k0 + lk) * DVP;
+      const float w = wj[k0 + lk];
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        acc[s] = __builtin_amdgcn_mfma_f32_32x32x2f32(to_float(krow[k_at[s]]), to_float(vrow[v_at[s]]) * w, acc[s], 0, 0, 0);
+    }
   }
-  const size_t per = (size_t)dk * dv;
-  const size_t at = (((size_t)b * n_seg + c) * H + h) * per;
-  const float* S_old = state + ((size_t)slot * H + h) * per;
-  const float fade = pwh[n];
+  const size_t at = (((size_t)b * n_seg + c) * H + h) * (size_t)dk * dv;
   const bool whole = (dk & 31) == 0 && (dv & 31) == 0;
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
@@ -1090,24 +1116,38 @@ __global__ void __launch_bounds__(LC_THREADS)
     if (t < tiles) {
       const int tr = t / NV, tc = t - tr * NV;
       const int col = tc * 32 + lr, i0 = tr * 32 + 4 * lk;
-      const size_t o = (size_t)i0 * dv + col;
-      float* end_p = seg_end + at + o;
+      float* end_p = seg_end + at + (size_t)i0 * dv + col;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int di = 8 * (r / 4) + (r & 3);
-        if (whole || (i0 + di < dk && col < dv)) {
-          float v = acc[s][r];
-          if (c == 0) {
-            const float old = S_old[o + (size_t)di * dv];
-            seg_start[at + o + (size_t)di * dv] = old;
-            v = fmaf(fade, old, v);
-          }
-          end_p[(size_t)di * dv] = v;
-        }
+        if (whole || (i0 + di < dk && col < dv)) end_p[(size_t)di * dv] = acc[s][r];
       }
     }
   }
-  for (int i = threadIdx.x; i < dk; i += LC_THREADS) seg_decay[(((size_t)b * n_seg + c) * H + h) * dk + i] = fade;
+}
+
+// From chunk to chunk: start[0] is the sequence's state, start[c + 1] = a^(tokens of chunk c) start[c] + end[c]; what
+// comes out behind the last chunk is the sequence's new state.
+__global__ void lc_carry_kernel(const float* __restrict__ seg_end, float* __restrict__ seg_start, float* __restrict__ state,
+                                const float* __restrict__ pw, const int* __restrict__ cu_seqlens,
+                                const int* __restrict__ seq_slots, int H, int dk, int dv, int n_seg) {
+  const int b = blockIdx.y;
+  const int slot = seq_slots[b];
+  const int n_new = cu_seqlens[b + 1] - cu_seqlens[b];
+  if (slot < 0 || n_new <= 0) return;
+  const int ns = (n_new + LC_CHUNK - 1) / LC_CHUNK;
+  const size_t per_head = (size_t)dk * dv, per = (size_t)H * per_head;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < per; e += (size_t)gridDim.x * blockDim.x) {
+    const float* pwh = pw + (e / per_head) * (LC_CHUNK + 1);
+    const float whole = pwh[LC_CHUNK], last = pwh[n_new - (ns - 1) * LC_CHUNK];
+    float S = state[(size_t)slot * per + e];
+    for (int c = 0; c < ns; ++c) {
+      const size_t at = ((size_t)b * n_seg + c) * per + e;
+      seg_start[at] = S;
+      S = fmaf(c + 1 < ns ? whole : last, S, seg_end[at]);
+    }
+    state[(size_t)slot * per + e] = S;
+  }
 }
 
 template <typename TA>
@@ -1129,14 +1169,17 @@ __global__ void __launch_bounds__(LC_THREADS)
   TA* Ks = Qs + LC_CHUNK * SK;                                      // [64][SK]
   TA* Vs = Ks + LC_CHUNK * SK;                                      // [64][DVP]
   const TA* rows = proj + (size_t)(first + t0) * ld;
-  lc_stage<TA>(rows, ld, h * dk, dk, DKP, n, Qs, SK);
-  lc_stage<TA>(rows, ld, H * dk + h * dk, dk, DKP, n, Ks, SK);
-  lc_stage<TA>(rows, ld, 2 * H * dk + h * dv, dv, DVP, n, Vs, DVP);
+  {
+    LcOperands<TA, 3> op;
+    op.col0[0] = h * dk; op.width[0] = dk; op.WP[0] = DKP; op.row_ld[0] = SK; op.dst[0] = Qs;
+    op.col0[1] = H * dk + h * dk; op.width[1] = dk; op.WP[1] = DKP; op.row_ld[1] = SK; op.dst[1] = Ks;
+    op.col0[2] = 2 * H * dk + h * dv; op.width[2] = dv; op.WP[2] = DVP; op.row_ld[2] = DVP; op.dst[2] = Vs;
+    lc_stage<TA, 3>(rows, ld, n, op);
+  }
   if (threadIdx.x <= LC_CHUNK) pws[threadIdx.x] = pw[h * (LC_CHUNK + 1) + threadIdx.x];
   __syncthreads();
   const int wave = threadIdx.x / BLM_WAVE, lane = threadIdx.x & (BLM_WAVE - 1);
   const int lr = lane & 31, lk = lane >> 5;
-  const int depth_k = (dk + 1) & ~1;
   // scores of the three tiles at and below the diagonal, times the powers of the decay
   if (wave < 3) {
     const int ti = wave == 0 ? 0 : 1, tj = wave == 2 ? 1 : 0;
@@ -1145,9 +1188,11 @@ __global__ void __launch_bounds__(LC_THREADS)
     for (int r = 0; r < 16; ++r) sc[r] = 0.f;
     const TA* qrow = Qs + (ti * 32 + lr) * SK + lk;
     const TA* krow = Ks + (tj * 32 + lr) * SK + lk;
-#pragma unroll 8
-    for (int k0 = 0; k0 < depth_k; k0 += 2)
-      sc = __builtin_amdgcn_mfma_f32_32x32x2f32(to_float(qrow[k0]), to_float(krow[k0]), sc, 0, 0, 0);
+    for (int kb = 0; kb < DKP; kb += 2 * LC_STEPS) {
+#pragma unroll
+      for (int u = 0; u < LC_STEPS; ++u)
+        sc = __builtin_amdgcn_mfma_f32_32x32x2f32(to_float(qrow[kb + 2 * u]), to_float(krow[kb + 2 * u]), sc, 0, 0, 0);
+    }
     const int j = tj * 32 + lr;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -1174,12 +1219,20 @@ __global__ void __launch_bounds__(LC_THREADS)
     const TA* qrow = Qs + (ti * 32 + lr) * SK + lk;
     const float* s0 = S0 + min(ca, dv - 1);
     const float* s1 = S0 + min(cb, dv - 1);
-#pragma unroll 8
-    for (int k0 = 0; k0 < depth_k; k0 += 2) {
-      const size_t row = (size_t)min(k0 + lk, dk - 1) * dv;
-      const float a = to_float(qrow[k0]);
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s0[row], acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, s1[row], acc[1], 0, 0, 0);
+    for (int kb = 0; kb < DKP; kb += 2 * LC_STEPS) {
+      float sa[LC_STEPS], sb[LC_STEPS];
+#pragma unroll
+      for (int u = 0; u < LC_STEPS; ++u) {
+        const size_t row = (size_t)min(kb + 2 * u + lk, dk - 1) * dv;
+        sa[u] = s0[row];
+        sb[u] = s1[row];
+      }
+#pragma unroll
+      for (int u = 0; u < LC_STEPS; ++u) {
+        const float a = to_float(qrow[kb + 2 * u]);
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, sa[u], acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, sb[u], acc[1], 0, 0, 0);
+      }
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -1193,12 +1246,15 @@ __global__ void __launch_bounds__(LC_THREADS)
     const float* arow = As + (ti * 32 + lr) * LC_A_LD + lk;
     const TA* v0 = Vs + lk * DVP + ca;
     const TA* v1 = Vs + lk * DVP + cb;
-    const int depth = min((ti + 1) * 32, (n + 1) & ~1);
-#pragma unroll 8
-    for (int k0 = 0; k0 < depth; k0 += 2) {
-      const float a = arow[k0];
-      acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(v0[k0 * DVP]), acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(v1[k0 * DVP]), acc[1], 0, 0, 0);
+    const int depth = min((ti + 1) * 32, (n + 2 * LC_STEPS - 1) & ~(2 * LC_STEPS - 1));
+    for (int kb = 0; kb < depth; kb += 2 * LC_STEPS) {
+#pragma unroll
+      for (int u = 0; u < LC_STEPS; ++u) {
+        const int k0 = kb + 2 * u;
+        const float a = arow[k0];
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(v0[k0 * DVP]), acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, to_float(v1[k0 * DVP]), acc[1], 0, 0, 0);
+      }
     }
   }
 #pragma unroll
@@ -1246,18 +1302,18 @@ extern "C" int blm_lightning_chunks_init() {
 extern "C" int blm_lightning_chunks_supported(int dk, int dv) { return (dk >= 1 && dk <= LC_MAX && dv >= 1 && dv <= LC_MAX) ? 1 : 0; }
 
 // proj as for blm_gla_scan (queries, keys, values, output-gate logits); pw [H][65] float: powers 0 .. 64 of every head's
-// decay; n_seg: chunks of 64 tokens that cover the longest sequence of the step; seg_end, seg_start [B][n_seg][H][dk][dv],
-// seg_decay [B][n_seg][H][dk] float.  state is read and left updated; o_raw [T][H*dv] float; out [T][H*dv] in proj's type.
+// decay; n_seg: chunks of 64 tokens that cover the longest sequence of the step; seg_end, seg_start [B][n_seg][H][dk][dv]
+// float.  state is read and left updated; o_raw [T][H*dv] float; out [T][H*dv] in proj's type.
 // act_mode, norm_all, gate_mode as for blm_gla_scan (act_mode 1 activates proj's queries, keys and values in place).
 extern "C" int blm_lightning_chunks(void* proj, int dtype, int ld, const float* pw, const float* norm_w, float eps,
                                     float* state, float* o_raw, void* out, const int* cu_seqlens, const int* seq_slots, int T,
                                     int B, int H, int dk, int dv, int max_new, int n_seg, float* seg_end, float* seg_start,
-                                    float* seg_decay, int act_mode, int norm_all, int gate_mode, hipStream_t stream) {
+                                    int act_mode, int norm_all, int gate_mode, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && B > 0 && B <= 65535 && H > 0 && H <= 65535, "lightning_chunks: bad sizes T=%d B=%d H=%d", T, B, H);
   BLM_REQUIRE(blm_lightning_chunks_supported(dk, dv), "lightning_chunks: heads of %d x %d channels are not supported (up to %d)", dk, dv, LC_MAX);
   BLM_REQUIRE(ld >= 2 * H * dk + 2 * H * dv, "lightning_chunks: rows of %d are too short", ld);
   BLM_REQUIRE(dtype == BLM_F32 || dtype == BLM_BF16, "lightning_chunks: unsupported dtype %d", dtype);
-  BLM_REQUIRE(max_new >= 1 && n_seg >= 1 && (long long)n_seg * LC_CHUNK >= max_new && pw && seg_end && seg_start && seg_decay,
+  BLM_REQUIRE(max_new >= 1 && n_seg >= 1 && (long long)n_seg * LC_CHUNK >= max_new && pw && seg_end && seg_start,
               "lightning_chunks: %d chunks do not cover %d tokens, or no workspace", n_seg, max_new);
   BLM_REQUIRE((act_mode == 0 || act_mode == 1) && (gate_mode == 1 || gate_mode == 2), "lightning_chunks: unknown activation %d or gate %d", act_mode, gate_mode);
   int dev = -1;
@@ -1282,17 +1338,17 @@ extern "C" int blm_lightning_chunks(void* proj, int dtype, int ld, const float* 
   }
   const dim3 grid((unsigned)n_seg, (unsigned)H, (unsigned)B);
   if (dtype == BLM_F32)
-    hipLaunchKernelGGL(lc_state_kernel<float>, grid, dim3(LC_THREADS), lds_a, stream, (const float*)proj, ld, pw, state,
-                       seg_end, seg_start, seg_decay, cu_seqlens, seq_slots, H, dk, dv, n_seg);
+    hipLaunchKernelGGL(lc_state_kernel<float>, grid, dim3(LC_THREADS), lds_a, stream, (const float*)proj, ld, pw, seg_end,
+                       cu_seqlens, seq_slots, H, dk, dv, n_seg);
   else
-    hipLaunchKernelGGL(lc_state_kernel<bf16>, grid, dim3(LC_THREADS), lds_a, stream, (const bf16*)proj, ld, pw, state,
-                       seg_end, seg_start, seg_decay, cu_seqlens, seq_slots, H, dk, dv, n_seg);
+    hipLaunchKernelGGL(lc_state_kernel<bf16>, grid, dim3(LC_THREADS), lds_a, stream, (const bf16*)proj, ld, pw, seg_end,
+                       cu_seqlens, seq_slots, H, dk, dv, n_seg);
   BLM_LAUNCH_CHECK("lc_state");
   const size_t per = (size_t)H * dk * dv;
   const unsigned cb = (unsigned)((per + 255) / 256 < 1024 ? (per + 255) / 256 : 1024);
-  hipLaunchKernelGGL(gla_carry_kernel, dim3(cb, B), dim3(256), 0, stream, seg_end, seg_decay, seg_start, state, cu_seqlens,
-                     seq_slots, H, dk, dv, n_seg, LC_CHUNK);
-  BLM_LAUNCH_CHECK("gla_carry");
+  hipLaunchKernelGGL(lc_carry_kernel, dim3(cb, B), dim3(256), 0, stream, seg_end, seg_start, state, pw, cu_seqlens, seq_slots, H,
+                     dk, dv, n_seg);
+  BLM_LAUNCH_CHECK("lc_carry");
   if (dtype == BLM_F32)
     hipLaunchKernelGGL(lc_out_kernel<float>, grid, dim3(LC_THREADS), lds_c, stream, (const float*)proj, ld, pw, seg_start,
                        o_raw, cu_seqlens, seq_slots, H, dk, dv, n_seg);
