@@ -255,6 +255,11 @@ def build(verbose=True, jobs=None, with_ref=False):
                         q.kill()
                     raise RuntimeError(f"hipcc failed on {s}:\n{out}")
                 log(f"  {s} done ({time.time() - t0:.0f} s)")
+                # a loop that the compiler was asked to unroll and did not (it refuses around matrix instructions when
+                # the trip count is only known at run time) costs a kernel most of its speed: say so
+                for line in out.splitlines():
+                    if "-Wpass-failed" in line:
+                        log(f"  {s}: {line.strip()}")
         if running and time.time() - last_note > 15:
             log(f"  still compiling: {', '.join(sorted(running))} ({time.time() - t0:.0f} s)")
             last_note = time.time()
