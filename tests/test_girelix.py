@@ -608,17 +608,18 @@ def test_routing_and_adding_kernels_against_the_plain_functions():
         assert np.abs(got - want).max() < 1e-5, (E, I, count, keep, top)
         assert np.allclose(got.sum(1), 1.0, atol=1e-5)
     # sublayer results into the residual, each with its coefficients: float planes, one bfloat16 plane, a factor per
-    # token read with a stride, a term without coefficients
-    T, D = 5, 20
-    h = rng.standard_normal((T, D))
-    a, b, c, d = rng.standard_normal((2, T, D)), rng.standard_normal((T, D)), rng.standard_normal((1, T, D)), rng.standard_normal((T, D))
-    ca, cb = rng.standard_normal(D), rng.standard_normal(D)
-    rows = rng.standard_normal((T, 3))
-    hd, rows_dev = f32(h), f32(rows)
-    b16 = f32(b).bfloat16()
-    ops.scaled_add(hd, [(f32(a), f32(ca), None), (b16, f32(cb), rows_dev[:, 2]), (f32(c), None, None), (f32(d), None, rows_dev[:, 0])])
-    want = h + ca * a.sum(0) + cb * rows[:, 2:3] * b16.double().cpu().numpy() + c[0] + rows[:, 0:1] * d
-    assert np.abs(hd.double().cpu().numpy() - want).max() < 1e-5
+    # token read with a stride, a term without coefficients; widths that are and are not a multiple of four (four
+    # channels per lane, or one)
+    for T, D in ((5, 20), (7, 18), (300, 64)):
+        h = rng.standard_normal((T, D))
+        a, b, c, d = rng.standard_normal((2, T, D)), rng.standard_normal((T, D)), rng.standard_normal((1, T, D)), rng.standard_normal((T, D))
+        ca, cb = rng.standard_normal(D), rng.standard_normal(D)
+        rows = rng.standard_normal((T, 3))
+        hd, rows_dev = f32(h), f32(rows)
+        b16 = f32(b).bfloat16()
+        ops.scaled_add(hd, [(f32(a), f32(ca), None), (b16, f32(cb), rows_dev[:, 2]), (f32(c), None, None), (f32(d), None, rows_dev[:, 0])])
+        want = h + ca * a.sum(0) + cb * rows[:, 2:3] * b16.double().cpu().numpy() + c[0] + rows[:, 0:1] * d
+        assert np.abs(hd.double().cpu().numpy() - want).max() < 1e-5, (T, D)
 
 
 @pytest.mark.gpu
