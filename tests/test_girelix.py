@@ -530,7 +530,9 @@ def test_keys_are_turned_in_adjacent_pairs_and_kept_unturned_as_values(dtype):
 @pytest.mark.parametrize("H,dk,dv", [(3, 12, 20), (10, 4, 250), (2, 128, 128), (3, 70, 33)],
                          ids=["small", "norm_over_2500_lanes", "largest_chunked_heads", "odd"])
 @pytest.mark.parametrize("form", ["scan", "chunks"])
-def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv, form):
+@pytest.mark.parametrize("news,slots", [([300, 40, 1], [2, 0, 3]), ([64, 65, 63, 128, 129, 1, 8, 2], [5, 0, 3, 8, 2, 7, 4, 6])],
+                         ids=["long", "chunk_edges"])
+def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv, form, news, slots):
     """Three sequences in one step: a long prompt (walked in segments, or in chunks of 64 tokens whose last one is not
     full), a continuation from a state, one token from a state; heads that forget at once, slowly and never; a state slot
     that is not in the step stays as it was.  The recurrence is written out here once more, on rows that stand for the
@@ -544,9 +546,8 @@ def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv, form):
     bf = lambda a: torch.from_numpy(np.asarray(a, dtype=np.float32)).to(dtype).double().numpy()
     W = {"r.norm": rng.uniform(0.5, 1.5, H * dv)}
     act = lambda z: bf(P.silu(z))            # the activations are rounded to the rows' type
-    news, slots = [300, 40, 1], [2, 0, 3]
-    states = rng.standard_normal((4, H, dk, dv))
-    states[2] = 0.0
+    states = rng.standard_normal((max(slots) + 1, H, dk, dv))      # slot 1 belongs to no sequence of the step
+    states[slots[0]] = 0.0
     width = 2 * H * dk + 2 * H * dv
     proj = bf(rng.standard_normal((sum(news), width)))
     # the plain function projects its input with identities: one input per projection
@@ -562,7 +563,7 @@ def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv, form):
                 o[t, hd] = S[hd].T @ act(q[t].reshape(H, dk)[hd])
         want.append((P.rms_norm(o.reshape(n, H * dv), W["r.norm"], 1e-5) * P.sigmoid(gl), S))
         at += n
-    step = _Step(news, [0, 77, 500], slots, dev)
+    step = _Step(news, [0, 77, 500, 3, 64, 640, 1, 0][:len(news)], slots, dev)
     f32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.float32, device=dev)
     state_dev = f32(states)
     T = sum(news)
@@ -574,7 +575,8 @@ def test_fading_state_kernel_against_the_plain_function(dtype, H, dk, dv, form):
                              activation="silu", norm_all=True, gate="sigmoid")
     else:
         ops.gla_scan(torch.from_numpy(proj).to(dev, dtype), None, None, None, f32(W["r.norm"]), 1e-5, state_dev,
-                     torch.zeros(T, H * dv, dtype=torch.float32, device=dev), out, step, H, dk, dv, segments=(3, 104),
+                     torch.zeros(T, H * dv, dtype=torch.float32, device=dev), out, step, H, dk, dv,
+                     segments=(3, 104) if max(news) > 200 else (2, 72),
                      fixed_decay=f32(np.repeat(r["decay"], dk)), activation="silu", q_scale=1.0, norm_all=True, gate="sigmoid")
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     at = 0
