@@ -110,6 +110,8 @@ class GirelixConfig:
             if vdim != dim:
                 raise ConfigError(f"config.json: {lw}.vdim must equal dim: the values of this attention are its keys")
             rot = l.get("rot")
+            if isinstance(rot, dict) and rot.get("dims") == 0 and not isinstance(rot.get("dims"), bool):
+                rot = None      # no lanes turn
             rot_dims = _get(rot, "dims", int, lw + ".rot") if rot is not None else 0
             if rot_dims % 2 or rot_dims > dim:
                 raise ConfigError(f"config.json: {lw}.rot.dims must be even and at most dim")

@@ -688,9 +688,8 @@ __global__ void __launch_bounds__(256)
 extern "C" int blm_moe_route_grouped(const float* logits, int ld, const float* correction, int E, int n_identity, int groups,
                                      int keep, int top, float* weights, int T, hipStream_t stream) {
   const int N = E + n_identity;
-  BLM_REQUIRE(T > 0 && E >= 0 && n_identity >= 0 && N >= 1 && N <= PB_MAX_ROUTED && ld >= N && top >= 1 && top <= PB_MAX_TOP,
-              "moe_route_grouped: bad sizes T=%d experts=%d+%d (at most %d) top=%d (at most %d)", T, E, n_identity,
-              PB_MAX_ROUTED, top, PB_MAX_TOP);
+  BLM_REQUIRE(T > 0 && E >= 0 && n_identity >= 0 && N >= 1 && N <= PB_MAX_ROUTED && ld >= N && top >= 1 && top <= N,
+              "moe_route_grouped: bad sizes T=%d experts=%d+%d (at most %d) top=%d", T, E, n_identity, PB_MAX_ROUTED, top);
   BLM_REQUIRE(groups <= 1 || (N % groups == 0 && keep >= 1 && keep <= groups), "moe_route_grouped: %d experts in %d groups, %d kept",
               N, groups, keep);
   BLM_REQUIRE(top <= (groups > 1 ? keep * (N / groups) : N), "moe_route_grouped: top=%d is more than the kept groups hold", top);

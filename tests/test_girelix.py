@@ -156,6 +156,9 @@ def test_config_is_read_and_refused_by_key():
         at[path[-1]] = value
         with pytest.raises(ConfigError, match=word):
             arch.read_config(bad)
+    none = json.loads(json.dumps(MIXED))
+    none["layers"][0]["mixer"]["left"]["rot"] = dict(base=10000.0, dims=0)      # no lanes turn
+    assert arch.read_config(none).layers[0].mixer.left.rot_dims == 0
     one = json.loads(json.dumps(MIXED))
     one["layers"][0]["mixer"]["right"]["decay"] = 0.75      # one number stands for every head
     assert arch.read_config(one).layers[0].mixer.right.decay == (0.75,) * one["layers"][0]["mixer"]["right"]["heads"]
@@ -593,7 +596,7 @@ def test_routing_and_adding_kernels_against_the_plain_functions():
     dev = "cuda"
     rng = np.random.default_rng(2)
     f32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.float32, device=dev)
-    for E, I, count, keep, top in ((5, 3, 4, 2, 3), (6, 0, 1, 1, 2), (1, 5, 3, 3, 6), (9, 3, 6, 1, 2), (4, 4, 2, 1, 4), (7, 0, 0, 1, 7)):
+    for E, I, count, keep, top in ((5, 3, 4, 2, 3), (6, 0, 1, 1, 2), (1, 5, 3, 3, 6), (9, 3, 6, 1, 2), (4, 4, 2, 1, 4), (7, 0, 0, 1, 7), (30, 10, 4, 3, 20), (100, 28, 8, 4, 9)):
         N, T = E + I, 257
         logits = rng.standard_normal((T, N + 3)) * 2              # three columns of padding behind the logits
         correction = rng.standard_normal(N) * 0.3
