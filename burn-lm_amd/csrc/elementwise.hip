@@ -85,21 +85,32 @@ extern "C" int blm_embed_gather_from(const void* table, int table_dtype, const i
 //   out[i] = v / sqrt(mean(v^2) + eps) * gamma;     r = rows ? rows[i] : i
 //   delta: n_planes planes of [T, D], in the activation dtype or float (partial products of a
 //   matrix product whose K was cut over blocks; summed here in plane order).
+//   GATED: the summed delta joins as mult * delta * sigmoid(gate_z[r] + gate_b) (gate_z [T, D] in the activation
+//   dtype, gate_b [D] float or null): a sublayer's result behind a gate that was projected from the sublayer's input.
 // ---------------------------------------------------------------------------------------
-template <typename TA, typename TG, typename TD>
+__device__ __forceinline__ float gate_sigmoid(float z) { return 1.0f / (1.0f + __expf(-z)); }
+template <typename TA, typename TG, typename TD, bool GATED>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_planes,
                                    size_t plane_stride, const TG* __restrict__ gamma, TA* __restrict__ out,
-                                   const int* __restrict__ rows, int D, float eps, int write_h) {
+                                   const int* __restrict__ rows, int D, float eps, int write_h,
+                                   const TA* __restrict__ gate_z, const float* __restrict__ gate_b, float mult) {
   __shared__ float red[17];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
   float* hr = h + (size_t)r * D;
   const TD* dr = delta ? delta + (size_t)r * D : nullptr;
+  const TA* zr = GATED ? gate_z + (size_t)r * D : nullptr;
   float ss = 0.f;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float v = hr[d];
     if (dr) {
-      for (int p = 0; p < n_planes; ++p) v += to_float(dr[p * plane_stride + d]);
+      if (GATED) {
+        float a = 0.f;
+        for (int p = 0; p < n_planes; ++p) a += to_float(dr[p * plane_stride + d]);
+        v += mult * a * gate_sigmoid(to_float(zr[d]) + (gate_b ? gate_b[d] : 0.f));
+      } else {
+        for (int p = 0; p < n_planes; ++p) v += to_float(dr[p * plane_stride + d]);
+      }
       if (write_h) hr[d] = v;
     }
     ss += v * v;
@@ -109,8 +120,15 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   TA* o = out + (size_t)i * D;
   for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float v = hr[d];
-    if (dr && !write_h)
-      for (int p = 0; p < n_planes; ++p) v += to_float(dr[p * plane_stride + d]);
+    if (dr && !write_h) {
+      if (GATED) {
+        float a = 0.f;
+        for (int p = 0; p < n_planes; ++p) a += to_float(dr[p * plane_stride + d]);
+        v += mult * a * gate_sigmoid(to_float(zr[d]) + (gate_b ? gate_b[d] : 0.f));
+      } else {
+        for (int p = 0; p < n_planes; ++p) v += to_float(dr[p * plane_stride + d]);
+      }
+    }
     o[d] = from_float<TA>(v * inv * to_float(gamma[d]));
   }
 }
@@ -157,11 +175,12 @@ __device__ __forceinline__ void store4<bf16>(bf16* p, const float* v) {
   *reinterpret_cast<uint2*>(p) = r;
 }
 
-template <typename TA, typename TG, typename TD, int ITERS>
+template <typename TA, typename TG, typename TD, int ITERS, bool GATED>
 __global__ void __launch_bounds__(512)
     add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta, int n_planes, size_t plane_stride,
                            const TG* __restrict__ gamma, TA* __restrict__ out, const int* __restrict__ rows, int D,
-                           float eps, int write_h) {
+                           float eps, int write_h, const TA* __restrict__ gate_z, const float* __restrict__ gate_b,
+                           float mult) {
   __shared__ float red[17];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
@@ -185,6 +204,19 @@ __global__ void __launch_bounds__(512)
     const int d = (it * blockDim.x + threadIdx.x) * 4;
     if (d < D) {
       load4<float>(hr + d, v[it]);
+      // GATED: the planes are summed from zero, and the sum joins the row behind its gate
+      float base[4] = {0.f, 0.f, 0.f, 0.f}, factor[4] = {1.f, 1.f, 1.f, 1.f};
+      if (GATED && dr) {
+        float zg[4], bg[4] = {0.f, 0.f, 0.f, 0.f};
+        load4<TA>(gate_z + (size_t)r * D + d, zg);
+        if (gate_b) load4<float>(gate_b + d, bg);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          base[e] = v[it][e];
+          v[it][e] = 0.f;
+          factor[e] = mult * gate_sigmoid(zg[e] + bg[e]);
+        }
+      }
       if (dr) {
         // four planes at a time: their loads are issued together (a loop that loads and adds plane
         // by plane waits for memory once per plane), the adds keep the planes' order
@@ -218,6 +250,10 @@ __global__ void __launch_bounds__(512)
           }
         }
       }
+      if (GATED && dr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[it][e] = base[e] + factor[e] * v[it][e];
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e) ss += v[it][e] * v[it][e];
     }
@@ -246,18 +282,19 @@ __global__ void __launch_bounds__(512)
   }
 }
 
-template <typename TA, typename TG>
+template <typename TA, typename TG, bool GATED>
 static int launch_norm(float* h, const void* delta, int delta_dtype, int n_planes, size_t plane_stride,
                        const void* gamma, void* out, const int* rows, int n_out, int D, float eps, int write_h,
-                       hipStream_t stream) {
+                       const void* gate_z, const float* gate_b, float mult, hipStream_t stream) {
   dim3 grid(n_out), block(D >= 2048 ? 512 : 256);
   const bool aligned = D % 4 == 0 && plane_stride % 4 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
-                       ((uintptr_t)gamma % 16) == 0 && ((uintptr_t)delta % 16) == 0;
+                       ((uintptr_t)gamma % 16) == 0 && ((uintptr_t)delta % 16) == 0 && ((uintptr_t)gate_z % 16) == 0 &&
+                       ((uintptr_t)gate_b % 16) == 0;
   if (aligned && D <= 4 * (int)block.x * 4) {
     const int iters = (D + 4 * (int)block.x - 1) / (4 * (int)block.x);
 #define BLM_NV(TD, IT)                                                                                             \
-  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TA, TG, TD, IT>), grid, block, 0, stream, h, (const TD*)delta, n_planes, \
-                     plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h)
+  hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TA, TG, TD, IT, GATED>), grid, block, 0, stream, h, (const TD*)delta, n_planes, \
+                     plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h, (const TA*)gate_z, gate_b, mult)
     if (delta_dtype == BLM_F32) {
       if (iters == 1) BLM_NV(float, 1); else if (iters == 2) BLM_NV(float, 2); else BLM_NV(float, 4);
     } else {
@@ -268,13 +305,28 @@ static int launch_norm(float* h, const void* delta, int delta_dtype, int n_plane
     return 0;
   }
   if (delta_dtype == BLM_F32)
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TG, float>), grid, block, 0, stream, h, (const float*)delta, n_planes,
-                       plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h);
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TG, float, GATED>), grid, block, 0, stream, h, (const float*)delta, n_planes,
+                       plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h, (const TA*)gate_z, gate_b, mult);
   else
-    hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TG, bf16>), grid, block, 0, stream, h, (const bf16*)delta, n_planes,
-                       plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h);
+    hipLaunchKernelGGL((add_rmsnorm_kernel<TA, TG, bf16, GATED>), grid, block, 0, stream, h, (const bf16*)delta, n_planes,
+                       plane_stride, (const TG*)gamma, (TA*)out, rows, D, eps, write_h, (const TA*)gate_z, gate_b, mult);
   BLM_LAUNCH_CHECK("add_rmsnorm");
   return 0;
+}
+
+template <bool GATED>
+static int norm_by_dtype(float* h, const void* delta, int delta_dtype, int n_planes, long long plane_stride,
+                         const void* gamma, int gamma_dtype, void* out, int act_dtype, const int* rows, int n_out, int D,
+                         float eps, int write_h, const void* gate_z, const float* gate_b, float mult, hipStream_t stream) {
+  if (act_dtype == BLM_F32 && gamma_dtype == BLM_F32)
+    return launch_norm<float, float, GATED>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, gate_z, gate_b, mult, stream);
+  if (act_dtype == BLM_BF16 && gamma_dtype == BLM_BF16)
+    return launch_norm<bf16, bf16, GATED>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, gate_z, gate_b, mult, stream);
+  if (act_dtype == BLM_BF16 && gamma_dtype == BLM_F32)
+    return launch_norm<bf16, float, GATED>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, gate_z, gate_b, mult, stream);
+  if (act_dtype == BLM_F32 && gamma_dtype == BLM_BF16)
+    return launch_norm<float, bf16, GATED>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, gate_z, gate_b, mult, stream);
+  return blm_fail("add_rmsnorm: unsupported dtypes act=%d gamma=%d", act_dtype, gamma_dtype);
 }
 
 extern "C" int blm_add_rmsnorm(float* h, const void* delta, int delta_dtype, int n_planes, long long plane_stride,
@@ -284,15 +336,21 @@ extern "C" int blm_add_rmsnorm(float* h, const void* delta, int delta_dtype, int
   BLM_REQUIRE(delta == nullptr || (n_planes >= 1 && n_planes <= 64 && plane_stride >= 0),
               "add_rmsnorm: bad planes %d", n_planes);
   BLM_REQUIRE(delta == nullptr || delta_dtype == BLM_F32 || delta_dtype == BLM_BF16, "add_rmsnorm: delta dtype %d", delta_dtype);
-  if (act_dtype == BLM_F32 && gamma_dtype == BLM_F32)
-    return launch_norm<float, float>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, stream);
-  if (act_dtype == BLM_BF16 && gamma_dtype == BLM_BF16)
-    return launch_norm<bf16, bf16>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, stream);
-  if (act_dtype == BLM_BF16 && gamma_dtype == BLM_F32)
-    return launch_norm<bf16, float>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, stream);
-  if (act_dtype == BLM_F32 && gamma_dtype == BLM_BF16)
-    return launch_norm<float, bf16>(h, delta, delta_dtype, n_planes, plane_stride, gamma, out, rows, n_out, D, eps, write_h, stream);
-  return blm_fail("add_rmsnorm: unsupported dtypes act=%d gamma=%d", act_dtype, gamma_dtype);
+  return norm_by_dtype<false>(h, delta, delta_dtype, n_planes, plane_stride, gamma, gamma_dtype, out, act_dtype, rows, n_out, D,
+                              eps, write_h, nullptr, nullptr, 1.0f, stream);
+}
+
+// The same where the delta joins behind a gate: h[r] += mult * delta[r] * sigmoid(gate_z[r] + gate_b).
+extern "C" int blm_add_gated_rmsnorm(float* h, const void* delta, int delta_dtype, int n_planes, long long plane_stride,
+                                     const void* gate_z, const float* gate_b, float mult, const void* gamma,
+                                     int gamma_dtype, void* out, int act_dtype, const int* rows, int n_out, int D,
+                                     float eps, int write_h, hipStream_t stream) {
+  BLM_REQUIRE(n_out > 0 && D > 0, "add_gated_rmsnorm: bad sizes n=%d D=%d", n_out, D);
+  BLM_REQUIRE(delta && gate_z && n_planes >= 1 && n_planes <= 64 && plane_stride >= 0,
+              "add_gated_rmsnorm: needs a delta of 1 to 64 planes and its gate, got %d planes", n_planes);
+  BLM_REQUIRE(delta_dtype == BLM_F32 || delta_dtype == BLM_BF16, "add_gated_rmsnorm: delta dtype %d", delta_dtype);
+  return norm_by_dtype<true>(h, delta, delta_dtype, n_planes, plane_stride, gamma, gamma_dtype, out, act_dtype, rows, n_out, D,
+                             eps, write_h, gate_z, gate_b, mult, stream);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -13,7 +13,7 @@
 
 // ---------------------------------------------------------------------------------------
 // down [T][ld_down]: R latent lanes then Dr key lanes.  q [T][ld_q], head h at h * (dn + Dr).  cos_sin [positions][half_t]
-// (cos, sin), of which the first rot/2 pairs turn lanes (i, i + rot/2) of the Dr part.
+// (cos, sin), of which the first rot/2 pairs turn lanes (i, i + rot/2) of the Dr part, or (adjacent) lanes (2i, 2i + 1).
 // qabs [T][H][R + Dr] (float or the cache's type) gets the rotated query parts at lane R.  vcache (may be null):
 // pages [R][page] that receive the latent transposed, for the matrix-core attention.
 // ---------------------------------------------------------------------------------------
@@ -23,7 +23,7 @@ __global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, co
                                     int half_t, int rot, TQ* __restrict__ qabs, TA* __restrict__ kcache, TA* __restrict__ vcache,
                                     const int* __restrict__ positions, const int* __restrict__ token_seq,
                                     const int* __restrict__ block_table, int table_width, int page_size, int R, int Dr,
-                                    int write_kv) {
+                                    int write_kv, int adjacent) {
   __shared__ float red[17];
   const int t = blockIdx.x;
   const int b = token_seq[t];
@@ -37,10 +37,11 @@ __global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, co
     const TA* src = q + (size_t)t * ld_q + (size_t)h * (dn + Dr) + dn;
     float v = to_float(src[d]);
     if (d < rot) {
-      const int pair = d < half ? d : d - half;
+      const bool first = adjacent ? !(d & 1) : d < half;
+      const int pair = adjacent ? d >> 1 : (d < half ? d : d - half);
       const float2 c = cs[pair];
-      const float other = to_float(src[d < half ? d + half : d - half]);
-      v = d < half ? v * c.x - other * c.y : v * c.x + other * c.y;
+      const float other = to_float(src[adjacent ? d ^ 1 : (d < half ? d + half : d - half)]);
+      v = first ? v * c.x - other * c.y : v * c.x + other * c.y;
     }
     qabs[((size_t)t * H + h) * (R + Dr) + R + d] = from_float<TQ>(v);
   }
@@ -63,10 +64,11 @@ __global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, co
   for (int d = threadIdx.x; d < Dr; d += blockDim.x) {
     float v = to_float(row[R + d]);
     if (d < rot) {
-      const int pair = d < half ? d : d - half;
+      const bool first = adjacent ? !(d & 1) : d < half;
+      const int pair = adjacent ? d >> 1 : (d < half ? d : d - half);
       const float2 c = cs[pair];
-      const float other = to_float(row[R + (d < half ? d + half : d - half)]);
-      v = d < half ? v * c.x - other * c.y : v * c.x + other * c.y;
+      const float other = to_float(row[R + (adjacent ? d ^ 1 : (d < half ? d + half : d - half))]);
+      v = first ? v * c.x - other * c.y : v * c.x + other * c.y;
     }
     dst[R + d] = from_float<TA>(v);
   }
@@ -75,20 +77,53 @@ __global__ void latent_write_kernel(const TA* __restrict__ down, int ld_down, co
 extern "C" int blm_latent_write(const void* down, int ld_down, const void* q, int ld_q, int dtype, int T, int H, int dn,
                                 const float* norm_w, float eps, const void* cos_sin, int half_t, int rot, void* qabs,
                                 int qabs_dtype, void* kcache, void* vcache, const int* positions, const int* token_seq, const int* block_table,
-                                int table_width, int page_size, int R, int Dr, int write_kv, hipStream_t stream) {
+                                int table_width, int page_size, int R, int Dr, int write_kv, int adjacent, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && H > 0 && dn >= 0 && R > 0 && Dr >= 0, "latent_write: bad sizes");
   BLM_REQUIRE(rot % 2 == 0 && rot >= 0 && rot <= Dr && rot / 2 <= half_t, "latent_write: %d turning lanes do not fit %d", rot, Dr);
   BLM_REQUIRE(page_size > 0 && table_width > 0 && ld_down >= R + Dr && ld_q >= H * (dn + Dr), "latent_write: bad geometry");
 #define BLM_LW(TA, TQ)                                                                                                  \
   hipLaunchKernelGGL((latent_write_kernel<TA, TQ>), dim3(T), dim3(256), 0, stream, (const TA*)down, ld_down, (const TA*)q, \
                      ld_q, H, dn, norm_w, eps, (const float2*)cos_sin, half_t, rot, (TQ*)qabs, (TA*)kcache, (TA*)vcache,  \
-                     positions, token_seq, block_table, table_width, page_size, R, Dr, write_kv)
+                     positions, token_seq, block_table, table_width, page_size, R, Dr, write_kv, adjacent)
   if (dtype == BLM_F32 && qabs_dtype == BLM_F32) BLM_LW(float, float);
   else if (dtype == BLM_BF16 && qabs_dtype == BLM_F32) BLM_LW(bf16, float);
   else if (dtype == BLM_BF16 && qabs_dtype == BLM_BF16) BLM_LW(bf16, bf16);
   else return blm_fail("latent_write: unsupported dtypes %d / %d", dtype, qabs_dtype);
 #undef BLM_LW
   BLM_LAUNCH_CHECK("latent_write");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// RMS norm of a slice of rows: out[t][d] = x[t][d] / sqrt(mean_d(x[t]^2) + eps) * w[d] for d < N; x [T][ld] (any row
+// stride), out [T][N] contiguous in x's type, w float.  Sums and scaling in float.  (A latent between two projections.)
+// ---------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void rmsnorm_rows_kernel(const TA* __restrict__ x, int ld, const float* __restrict__ w, float eps,
+                                    TA* __restrict__ out, int N) {
+  __shared__ float red[17];
+  const TA* row = x + (size_t)blockIdx.x * ld;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < N; d += blockDim.x) {
+    const float v = to_float(row[d]);
+    ss += v * v;
+  }
+  const float inv = 1.0f / sqrtf(block_sum<true>(ss, red) / (float)N + eps);
+  TA* o = out + (size_t)blockIdx.x * N;
+  for (int d = threadIdx.x; d < N; d += blockDim.x) o[d] = from_float<TA>(to_float(row[d]) * inv * w[d]);
+}
+
+extern "C" int blm_rmsnorm_rows(const void* x, int ld, int dtype, const float* w, float eps, void* out, int T, int N,
+                                hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && N > 0 && ld >= N, "rmsnorm_rows: bad sizes T=%d N=%d rows of %d", T, N, ld);
+  const int threads = N <= 64 ? 64 : N <= 128 ? 128 : 256;
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(rmsnorm_rows_kernel<float>, dim3(T), dim3(threads), 0, stream, (const float*)x, ld, w, eps, (float*)out, N);
+  else if (dtype == BLM_BF16)
+    hipLaunchKernelGGL(rmsnorm_rows_kernel<bf16>, dim3(T), dim3(threads), 0, stream, (const bf16*)x, ld, w, eps, (bf16*)out, N);
+  else
+    return blm_fail("rmsnorm_rows: unsupported dtype %d", dtype);
+  BLM_LAUNCH_CHECK("rmsnorm_rows");
   return 0;
 }
 

@@ -10,7 +10,7 @@ import torch
 
 from . import build as _build
 
-ABI_VERSION = 37
+ABI_VERSION = 38
 _lib = None
 _lock = threading.Lock()
 
@@ -45,7 +45,13 @@ _SIGNATURES = {
                              _c_int, _c_int, _c_int, _c_void_p],
     "blm_qkv_prepare": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_int,
                         _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                        _c_void_p],
+                        _c_void_p, _c_void_p],
+    "blm_sigmoid_gate": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_gelu_glu": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "blm_softcap": [_c_void_p, ctypes.c_longlong, _c_float, _c_void_p],
+    "blm_rmsnorm_rows": [_c_void_p, _c_int, _c_int, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_void_p],
+    "blm_add_gated_rmsnorm": [_c_void_p, _c_void_p, _c_int, _c_int, ctypes.c_longlong, _c_void_p, _c_void_p, _c_float,
+                              _c_void_p, _c_int, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "blm_scaled_add": [_c_void_p, _c_int, _c_int, _c_int] + [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int] * 4
                       + [_c_void_p],
     "blm_moe_route_grouped": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int,
@@ -65,7 +71,7 @@ _SIGNATURES = {
     "blm_xielu": [_c_void_p, _c_void_p, _c_int, ctypes.c_longlong, _c_float, _c_float, _c_void_p],
     "blm_latent_write": [_c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_float, _c_void_p,
                          _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
-                         _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "blm_latent_attn_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p],
     "blm_latent_attn_mfma_supported": [_c_int, _c_int],
@@ -274,11 +280,13 @@ def embed_gather_from(table, ids, source_rows, source_cell, out_h, scale=1.0):
     return out_h
 
 
-def add_rmsnorm(h, delta, gamma, eps, out, rows=None, write_h=True):
+def add_rmsnorm(h, delta, gamma, eps, out, rows=None, write_h=True, gate=None, gate_bias=None, mult=1.0):
     """v = h[r] (+ delta[r]); h[r] = v if write_h; out[i] = v / sqrt(mean(v^2) + eps) * gamma,
     with r = rows[i] if rows is given, else i.  h is the float32 residual stream.  delta: [T, D] in
-    out's dtype, or float32 [planes, T, D] whose planes are summed (partial matrix products)."""
-    _gpu(h, delta, gamma, out, rows)
+    out's dtype, or float32 [planes, T, D] whose planes are summed (partial matrix products).
+    gate ([T, D] in out's dtype; with gate_bias float32 [D] or None): the summed delta joins as
+    mult * delta * sigmoid(gate + gate_bias)."""
+    _gpu(h, delta, gamma, out, rows, gate, gate_bias)
     D = h.shape[1]
     n_out = out.shape[0]
     if h.dtype != torch.float32:
@@ -300,6 +308,16 @@ def add_rmsnorm(h, delta, gamma, eps, out, rows=None, write_h=True):
         _i32("rows", rows, n_out)
     elif n_out != h.shape[0]:
         raise KernelError("add_rmsnorm: out needs one row per row of h when rows is not given")
+    if gate is not None:
+        _contig("gate", gate)
+        if delta is None or gate.shape != h.shape or gate.dtype != out.dtype:
+            raise KernelError("add_rmsnorm: a gate comes with a delta, is [T, D] and of out's dtype")
+        if gate_bias is not None:
+            _f32("gate_bias", gate_bias, D)
+        _call("blm_add_gated_rmsnorm", h.data_ptr(), _ptr(delta), dcode, planes, stride, gate.data_ptr(), _ptr(gate_bias),
+              float(mult), gamma.data_ptr(), _code(gamma), out.data_ptr(), _code(out), _ptr(rows), n_out, D, float(eps),
+              1 if write_h else 0, _stream())
+        return out
     _call("blm_add_rmsnorm", h.data_ptr(), _ptr(delta), dcode, planes, stride, gamma.data_ptr(), _code(gamma),
           out.data_ptr(), _code(out), _ptr(rows), n_out, D, float(eps), 1 if write_h else 0, _stream())
     return out
@@ -884,14 +902,14 @@ def xielu(z, out, a_pos, a_neg):
 # ------------------------------------------------------------------------------------------
 # attention over a shared latent
 def latent_write(down, q, norm_w, eps, cos_sin, rot, qabs, kcache, step, block_table, page_size, H, dn, R, Dr,
-                 write_kv=True, vcache=None):
+                 write_kv=True, vcache=None, adjacent=False):
     """down [T, >= R + Dr]: latent lanes then the shared key lanes; q [T, H * (dn + Dr)].  The latent is RMS-normed
     (norm_w, eps), the first `rot` of the Dr key lanes are turned by the token's position (pairs half of rot
-    apart; cos_sin float32 [positions, n, 2]), and the row [latent | key lanes] goes into the token's place of the
+    apart, or adjacent lanes 2i and 2i + 1; cos_sin float32 [positions, n, 2]), and the row [latent | key lanes] goes into the token's place of the
     key pages [pages, 1, page, R + Dr].  The queries' Dr lanes are turned alike into qabs[:, :, R:] (float32
     [T, H, R + Dr], or the cache's dtype).  vcache: pages [pages, 1, R, page] that get the latent transposed."""
     _gpu(down, q, norm_w, cos_sin, qabs, kcache, block_table, vcache)
-    T = down.shape[0]
+    T = q.shape[0]
     _contig("cos_sin", cos_sin); _contig("kcache", kcache); _contig("qabs", qabs)
     _f32("norm_w", norm_w, R)
     if qabs.numel() != T * H * (R + Dr) or qabs.dtype not in (torch.float32, kcache.dtype):
@@ -900,6 +918,12 @@ def latent_write(down, q, norm_w, eps, cos_sin, rot, qabs, kcache, step, block_t
         _contig("vcache", vcache)
         if tuple(vcache.shape) != (kcache.shape[0], 1, R, page_size) or vcache.dtype != kcache.dtype:
             raise KernelError(f"latent_write: transposed latent pages {tuple(vcache.shape)} do not fit")
+    if down is None:
+        if write_kv:
+            raise KernelError("latent_write: rows to write need the down-projection's output")
+        down, ld_down = q, max(q.stride(0), R + Dr)      # never read
+    else:
+        ld_down = down.stride(0)
     if down.stride(1) != 1 or q.stride(1) != 1 or down.dtype != q.dtype or kcache.dtype != q.dtype:
         raise KernelError("latent_write: down, q and the cache must share a dtype, rows contiguous")
     if tuple(q.shape) != (T, H * (dn + Dr)) or tuple(kcache.shape[1:]) != (1, page_size, R + Dr):
@@ -907,10 +931,22 @@ def latent_write(down, q, norm_w, eps, cos_sin, rot, qabs, kcache, step, block_t
     if cos_sin.dtype != torch.float32 or cos_sin.dim() != 3 or cos_sin.shape[2] != 2 or cos_sin.shape[0] <= step.max_position:
         raise KernelError("latent_write: cos_sin must be float32 [positions, pairs, 2] and cover the step's positions")
     _i32("block_table", block_table)
-    _call("blm_latent_write", down.data_ptr(), down.stride(0), q.data_ptr(), q.stride(0), _code(q), T, H, dn, norm_w.data_ptr(),
+    _call("blm_latent_write", down.data_ptr(), ld_down, q.data_ptr(), q.stride(0), _code(q), T, H, dn, norm_w.data_ptr(),
           float(eps), cos_sin.data_ptr(), cos_sin.shape[1], rot, qabs.data_ptr(), _code(qabs), kcache.data_ptr(),
           _ptr(vcache), step.positions.data_ptr(), step.token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
-          R, Dr, 1 if write_kv else 0, _stream())
+          R, Dr, 1 if write_kv else 0, 1 if adjacent else 0, _stream())
+
+
+def rmsnorm_rows(x, w, eps, out):
+    """out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * w over the N lanes of out's rows; x [T, N] with any row stride (a
+    slice of a projection's rows), out [T, N] contiguous in x's dtype, w float32 [N]."""
+    _gpu(x, w, out)
+    T, N = out.shape
+    _contig("out", out); _f32("w", w, N)
+    if tuple(x.shape) != (T, N) or x.stride(1) != 1 or x.dtype != out.dtype:
+        raise KernelError("rmsnorm_rows: x is [T, N] with contiguous rows in out's dtype")
+    _call("blm_rmsnorm_rows", x.data_ptr(), x.stride(0), _code(x), w.data_ptr(), float(eps), out.data_ptr(), T, N, _stream())
+    return out
 
 
 def head_project(x, in_head, w, out, out_head, K=None):
@@ -1173,6 +1209,37 @@ def clamped_glu(gate_up, out, limit, alpha):
     return out
 
 
+def gelu_glu(gate_up, out):
+    """out = gelu_tanh(gate) * up; gate_up [T, 2 I]: gate columns, then up columns."""
+    _gpu(gate_up, out)
+    T, I = out.shape
+    _contig("gate_up", gate_up); _contig("out", out)
+    if tuple(gate_up.shape) != (T, 2 * I) or gate_up.dtype != out.dtype:
+        raise KernelError("gelu_glu: gate_up is [T, 2 I] in out's dtype")
+    _call("blm_gelu_glu", gate_up.data_ptr(), out.data_ptr(), _code(out), T, I, _stream())
+    return out
+
+
+def softcap(logits, cap):
+    """logits <- cap * tanh(logits / cap), in place on contiguous float32."""
+    _gpu(logits)
+    _contig("logits", logits)
+    if logits.dtype != torch.float32 or not cap > 0:
+        raise KernelError("softcap: float32 logits and a positive cap")
+    _call("blm_softcap", logits.data_ptr(), logits.numel(), float(cap), _stream())
+    return logits
+
+
+def sigmoid_gate(x, gate):
+    """x[t, c] *= sigmoid(gate[t, c]) in place; x [T, N] and gate [T, N] with contiguous rows of any stride, one dtype."""
+    _gpu(x, gate)
+    T, N = x.shape
+    if tuple(gate.shape) != (T, N) or x.stride(1) != 1 or gate.stride(1) != 1 or x.dtype != gate.dtype:
+        raise KernelError("sigmoid_gate: x and gate are [T, N] with contiguous rows in one dtype")
+    _call("blm_sigmoid_gate", x.data_ptr(), x.stride(0), gate.data_ptr(), gate.stride(0), _code(x), T, N, _stream())
+    return x
+
+
 def moe_route(logits, bias, n_experts, top, shared_col, weights):
     """weights [T, E + 1] float32: for each token the softmax over its `top` largest of (logits[:, :E] + bias) at the
     chosen experts' places and zero elsewhere; at E the sigmoid of logits[:, shared_col] (shared_col < 0: one)."""
@@ -1361,13 +1428,16 @@ def lightning_chunks(proj, powers, norm_w, eps, state, o_raw, out, step, H, dk, 
 
 
 def qkv_prepare(qkv, bias, cos_sin, rot, step, block_table, kcache, vcache, page_size, H, G, dk, dv, write_kv=True,
-                adjacent=False, values_are_keys=False):
+                adjacent=False, values_are_keys=False, q_scale=None):
     """Bias, rotation of the first `rot` lanes of every query and key head by the token's position (lane i with
     lane i + rot/2, or with adjacent lanes 2i and 2i + 1; cos_sin float32 [positions, >= rot/2, 2] rows of exactly
     rot/2 pairs), queries in place, rotated keys and values into the pages (key pages [pages, G, page, dk], value pages
     [pages, G, dv, page]).  write_kv False: qkv holds queries only and nothing is stored.  values_are_keys: the rows
-    hold no values; a token's values are its keys as projected, before the rotation (dv = dk)."""
-    _gpu(qkv, bias, cos_sin, block_table, kcache, vcache)
+    hold no values; a token's values are its keys as projected, before the rotation (dv = dk).  q_scale (float32 [H]
+    or None): query head h is multiplied by q_scale[h] behind the rotation."""
+    _gpu(qkv, bias, cos_sin, block_table, kcache, vcache, q_scale)
+    if q_scale is not None:
+        _f32("q_scale", q_scale, H)
     T = qkv.shape[0]
     if qkv.stride(1) != 1:
         raise KernelError("qkv_prepare: rows must be contiguous")
@@ -1390,7 +1460,8 @@ def qkv_prepare(qkv, bias, cos_sin, rot, step, block_table, kcache, vcache, page
     _call("blm_qkv_prepare", qkv.data_ptr(), _code(qkv), qkv.stride(0), _ptr(bias), _ptr(cos_sin) if rot else 0, rot,
           step.positions.data_ptr(), step.token_seq.data_ptr(), _ptr(block_table) if write_kv else 0,
           block_table.shape[1] if write_kv else 0, _ptr(kcache) if write_kv else 0, _ptr(vcache) if write_kv else 0,
-          page_size, T, H, G, dk, dv, 1 if write_kv else 0, 1 if adjacent else 0, 1 if values_are_keys else 0, _stream())
+          page_size, T, H, G, dk, dv, 1 if write_kv else 0, 1 if adjacent else 0, 1 if values_are_keys else 0, _ptr(q_scale),
+          _stream())
     return qkv
 
 

@@ -327,6 +327,79 @@ extern "C" int blm_clamped_glu(const void* gate_up, void* out, int dtype, int T,
 }
 
 // ---------------------------------------------------------------------------------------
+// Gated feed-forward activation with the tanh form of GELU on the gate branch:
+//   out = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) * u;   gate_up [T][2 I]: gate columns, then up columns.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float pb_gelu_tanh(float g) {
+  const float a = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+  // tanh(a) = 1 - 2 / (1 + e^(2a)): exact at both ends (e^(2a) -> inf gives 1, -> 0 gives -1)
+  const float th = 1.0f - 2.0f / (1.0f + __expf(2.0f * a));
+  return 0.5f * g * (1.0f + th);
+}
+
+template <typename TA>
+__global__ void gelu_glu_kernel(const TA* __restrict__ gate_up, TA* __restrict__ out, long long n, int I) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const long long t = e / I;
+    const int i = (int)(e - t * I);
+    const float g = to_float(gate_up[(size_t)t * 2 * I + i]);
+    const float u = to_float(gate_up[(size_t)t * 2 * I + I + i]);
+    out[e] = from_float<TA>(pb_gelu_tanh(g) * u);
+  }
+}
+
+__global__ void gelu_glu8_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, long long n8, int I8) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n8; e += stride) {
+    const long long t = e / I8;
+    const int i = (int)(e - t * I8);
+    const uint4 g4 = *reinterpret_cast<const uint4*>(gate_up + ((size_t)t * 2 * I8 + i) * 8);
+    const uint4 u4 = *reinterpret_cast<const uint4*>(gate_up + ((size_t)t * 2 * I8 + I8 + i) * 8);
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      r[k] = f32x2_to_bf16x2_bits(pb_gelu_tanh(pb_lo(gw[k])) * pb_lo(uw[k]), pb_gelu_tanh(pb_hi(gw[k])) * pb_hi(uw[k]));
+    *reinterpret_cast<uint4*>(out + (size_t)e * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+  }
+}
+
+extern "C" int blm_gelu_glu(const void* gate_up, void* out, int dtype, int T, int I, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && I > 0, "gelu_glu: bad sizes T=%d I=%d", T, I);
+  const long long n = (long long)T * I;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(gelu_glu_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)gate_up, (float*)out, n, I);
+  else if (dtype == BLM_BF16 && I % 8 == 0 && ((size_t)gate_up & 15) == 0 && ((size_t)out & 15) == 0) {
+    const long long n8 = n / 8;
+    const unsigned b8 = (unsigned)((n8 + 255) / 256 < 65535 ? (n8 + 255) / 256 : 65535);
+    hipLaunchKernelGGL(gelu_glu8_kernel, dim3(b8), dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out, n8, I / 8);
+  } else if (dtype == BLM_BF16)
+    hipLaunchKernelGGL(gelu_glu_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out, n, I);
+  else
+    return blm_fail("gelu_glu: unsupported dtype %d", dtype);
+  BLM_LAUNCH_CHECK("gelu_glu");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// Soft cap of float logits, in place: z <- cap * tanh(z / cap).
+// ---------------------------------------------------------------------------------------
+__global__ void softcap_kernel(float* __restrict__ z, long long n, float cap, float inv_cap) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) z[e] = cap * tanhf(z[e] * inv_cap);
+}
+
+extern "C" int blm_softcap(float* z, long long n, float cap, hipStream_t stream) {
+  BLM_REQUIRE(n > 0 && cap > 0.f, "softcap: bad sizes n=%lld cap=%g", n, (double)cap);
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  hipLaunchKernelGGL(softcap_kernel, dim3(blocks), dim3(256), 0, stream, z, n, cap, 1.0f / cap);
+  BLM_LAUNCH_CHECK("softcap");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
 // Routing of a mixture of experts.  logits [T][ld] float: E router logits, then (if shared) one logit of the
 // shared expert's gate; bias [E] is added.  The `top` largest logits are chosen (the lower index wins a tie);
 // their weights are the softmax over the chosen logits only.  weights [T][E + 1] float: an expert's weight or 0,

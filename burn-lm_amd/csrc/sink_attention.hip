@@ -21,14 +21,16 @@
 // qkv [T][ld]: queries at column 0 (H * dk), then (if keys are written) keys (G * dk) and values (G * dv).
 // bias [H*dk (+ G*dk + G*dv)] float or null.  cos_sin [positions][rot/2][2] float.  adjacent: pair i of the turning
 // lanes is (2i, 2i + 1) instead of (i, i + rot/2).  values_are_keys (dv = dk): there are no value columns; a token's
-// values are its keys as projected (with their bias), before the rotation.
+// values are its keys as projected (with their bias), before the rotation.  q_scale [H] float or null: every lane of
+// query head h is multiplied by q_scale[h] behind the rotation (a temperature per head: the scores are linear in it).
 // ---------------------------------------------------------------------------------------
 template <typename TA>
 __global__ void qkv_prepare_kernel(TA* __restrict__ qkv, int ld, const float* __restrict__ bias,
                                    const float* __restrict__ cos_sin, int rot, const int* __restrict__ positions,
                                    const int* __restrict__ token_seq, const int* __restrict__ block_table, int table_width,
                                    TA* __restrict__ kcache, TA* __restrict__ vcache, int page_size, int H, int G, int dk,
-                                   int dv, int write_kv, int adjacent, int values_are_keys) {
+                                   int dv, int write_kv, int adjacent, int values_are_keys,
+                                   const float* __restrict__ q_scale) {
   const int t = blockIdx.x;
   const int b = token_seq[t];
   if (b < 0) return;
@@ -48,12 +50,13 @@ __global__ void qkv_prepare_kernel(TA* __restrict__ qkv, int ld, const float* __
     const int head = e / per_head, i = e - head * per_head;
     const int col = head * dk;
     TA* krow = head >= H ? kcache + (((size_t)page * G + (head - H)) * page_size + in_page) * dk : nullptr;
+    const float f = (q_scale && head < H) ? q_scale[head] : 1.0f;
     if (i < half) {
       const int la = adjacent ? 2 * i : i, lb = adjacent ? 2 * i + 1 : i + half;
       float u = to_float(row[col + la]), v = to_float(row[col + lb]);
       if (bias) { u += bias[col + la]; v += bias[col + lb]; }
       const float c = cs[2 * i], s = cs[2 * i + 1];
-      const float ru = u * c - v * s, rv = v * c + u * s;
+      const float ru = (u * c - v * s) * f, rv = (v * c + u * s) * f;
       if (krow) { krow[la] = from_float<TA>(ru); krow[lb] = from_float<TA>(rv); }
       else { row[col + la] = from_float<TA>(ru); row[col + lb] = from_float<TA>(rv); }
     } else {
@@ -61,7 +64,7 @@ __global__ void qkv_prepare_kernel(TA* __restrict__ qkv, int ld, const float* __
       float u = to_float(row[col + lane]);
       if (bias) u += bias[col + lane];
       if (krow) krow[lane] = from_float<TA>(u);
-      else row[col + lane] = from_float<TA>(u);
+      else row[col + lane] = from_float<TA>(u * f);
     }
   }
   if (write_kv) {
@@ -79,7 +82,7 @@ __global__ void qkv_prepare_kernel(TA* __restrict__ qkv, int ld, const float* __
 extern "C" int blm_qkv_prepare(void* qkv, int dtype, int ld, const float* bias, const float* cos_sin, int rot,
                                const int* positions, const int* token_seq, const int* block_table, int table_width,
                                void* kcache, void* vcache, int page_size, int T, int H, int G, int dk, int dv, int write_kv,
-                               int adjacent, int values_are_keys, hipStream_t stream) {
+                               int adjacent, int values_are_keys, const float* q_scale, hipStream_t stream) {
   BLM_REQUIRE(T > 0 && H > 0 && G > 0 && dk > 0 && dv > 0, "qkv_prepare: bad sizes T=%d H=%d G=%d dk=%d dv=%d", T, H, G, dk, dv);
   BLM_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dk, "qkv_prepare: %d turning lanes of %d (even, at most the head size)", rot, dk);
   BLM_REQUIRE(!values_are_keys || dv == dk, "qkv_prepare: values that are the keys have the keys' head size, not %d", dv);
@@ -88,13 +91,66 @@ extern "C" int blm_qkv_prepare(void* qkv, int dtype, int ld, const float* bias, 
   BLM_REQUIRE(rot == 0 || cos_sin, "qkv_prepare: the table of angles is missing");
   if (dtype == BLM_F32)
     hipLaunchKernelGGL(qkv_prepare_kernel<float>, dim3(T), dim3(256), 0, stream, (float*)qkv, ld, bias, cos_sin, rot, positions,
-                       token_seq, block_table, table_width, (float*)kcache, (float*)vcache, page_size, H, G, dk, dv, write_kv, adjacent, values_are_keys);
+                       token_seq, block_table, table_width, (float*)kcache, (float*)vcache, page_size, H, G, dk, dv, write_kv, adjacent, values_are_keys, q_scale);
   else if (dtype == BLM_BF16)
     hipLaunchKernelGGL(qkv_prepare_kernel<bf16>, dim3(T), dim3(256), 0, stream, (bf16*)qkv, ld, bias, cos_sin, rot, positions,
-                       token_seq, block_table, table_width, (bf16*)kcache, (bf16*)vcache, page_size, H, G, dk, dv, write_kv, adjacent, values_are_keys);
+                       token_seq, block_table, table_width, (bf16*)kcache, (bf16*)vcache, page_size, H, G, dk, dv, write_kv, adjacent, values_are_keys, q_scale);
   else
     return blm_fail("qkv_prepare: unsupported dtype %d", dtype);
   BLM_LAUNCH_CHECK("qkv_prepare");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// Output gate: x[t][c] *= sigmoid(g[t][c]) for c < N, in float, rounded once.  x [T][ld_x], g [T][ld_g] (the gate's
+// columns of the projection's rows).
+// ---------------------------------------------------------------------------------------
+template <typename TA>
+__global__ void sigmoid_gate_kernel(TA* __restrict__ x, int ld_x, const TA* __restrict__ g, int ld_g, long long n, int N) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
+    const long long t = e / N;
+    const int c = (int)(e - t * N);
+    TA* px = x + (size_t)t * ld_x + c;
+    *px = from_float<TA>(to_float(*px) / (1.0f + __expf(-to_float(g[(size_t)t * ld_g + c]))));
+  }
+}
+
+// eight bfloat16 at a time (N, both row strides and both addresses multiples of eight elements)
+__global__ void sigmoid_gate8_kernel(bf16* __restrict__ x, int ld_x, const bf16* __restrict__ g, int ld_g, long long n8, int N8) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < n8; e += stride) {
+    const long long t = e / N8;
+    const int c = (int)(e - t * N8) * 8;
+    uint4* px = reinterpret_cast<uint4*>(x + (size_t)t * ld_x + c);
+    const uint4 xv = *px, gv = *reinterpret_cast<const uint4*>(g + (size_t)t * ld_g + c);
+    const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, gw[4] = {gv.x, gv.y, gv.z, gv.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float x0 = __uint_as_float(xw[k] << 16), x1 = __uint_as_float(xw[k] & 0xffff0000u);
+      const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+      r[k] = f32x2_to_bf16x2_bits(x0 / (1.0f + __expf(-g0)), x1 / (1.0f + __expf(-g1)));
+    }
+    *px = make_uint4(r[0], r[1], r[2], r[3]);
+  }
+}
+
+extern "C" int blm_sigmoid_gate(void* x, int ld_x, const void* g, int ld_g, int dtype, int T, int N, hipStream_t stream) {
+  BLM_REQUIRE(T > 0 && N > 0 && ld_x >= N && ld_g >= N, "sigmoid_gate: bad sizes T=%d N=%d rows of %d and %d", T, N, ld_x, ld_g);
+  const long long n = (long long)T * N;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+  if (dtype == BLM_F32)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, dim3(blocks), dim3(256), 0, stream, (float*)x, ld_x, (const float*)g, ld_g, n, N);
+  else if (dtype == BLM_BF16 && N % 8 == 0 && ld_x % 8 == 0 && ld_g % 8 == 0 && ((size_t)x & 15) == 0 && ((size_t)g & 15) == 0) {
+    const long long n8 = n / 8;
+    const unsigned b8 = (unsigned)((n8 + 255) / 256 < 65535 ? (n8 + 255) / 256 : 65535);
+    hipLaunchKernelGGL(sigmoid_gate8_kernel, dim3(b8), dim3(256), 0, stream, (bf16*)x, ld_x, (const bf16*)g, ld_g, n8, N / 8);
+  } else if (dtype == BLM_BF16)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (bf16*)x, ld_x, (const bf16*)g, ld_g, n, N);
+  else
+    return blm_fail("sigmoid_gate: unsupported dtype %d", dtype);
+  BLM_LAUNCH_CHECK("sigmoid_gate");
   return 0;
 }
 

@@ -1,3 +1,3 @@
 """Architectures: each module registers itself under the names its config.json uses."""
-from . import digasun, fuvirax, girelix, llama  # noqa: F401
+from . import bitonex, digasun, fuvirax, girelix, llama  # noqa: F401
 from .plan import LayerPlan, ModelPlan, Place  # noqa: F401

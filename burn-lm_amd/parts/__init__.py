@@ -1,13 +1,15 @@
 """Parts a model is assembled from, and their registration under kind names."""
 from .. import registry
 from .attention import Attention
-from .base import (Block, FeedForward, KVNeed, Mixer, Norm, Part, PartSpec, PositionEncoding, StateNeed,
+from .base import (Block, FeedForward, Gated, KVNeed, Mixer, Norm, Part, PartSpec, PositionEncoding, StateNeed,
                    TensorSpec)
 from .block import PreNormBlock
 from .channel_delta import ChannelDelta
 from .clamped_glu import ClampedGLU
 from .dense_xielu import DenseXielu
 from .embedding import Embedding, LMHead
+from .gated_residual import GatedPreNormBlock, GatedPreNormMixerBlock, ResidualGate
+from .gelu_glu import GeluGLU
 from .gla import GatedLinearAttention
 from .hgrn2 import HGRN2
 from .latent_attention import LatentAttention
@@ -52,3 +54,7 @@ registry.register_part("feed_forward", "grouped_experts", GroupedRoutedExperts)
 registry.register_part("connection", "layer_scale", LayerScale)
 registry.register_part("block", "parallel_scaled", ScaledParallelBlock)
 registry.register_part("block", "parallel_scaled_mixer_only", ScaledParallelMixerBlock)
+registry.register_part("connection", "residual_gate", ResidualGate)
+registry.register_part("block", "pre_norm_gated", GatedPreNormBlock)
+registry.register_part("block", "pre_norm_gated_mixer_only", GatedPreNormMixerBlock)
+registry.register_part("feed_forward", "gelu_glu", GeluGLU)

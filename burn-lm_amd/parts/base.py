@@ -12,7 +12,8 @@ Interfaces (all tensors live on the GPU; ``x`` is ``[tokens, width]`` in the act
 * ``Norm.add_norm(h, delta, rows=None, write_h=True) -> x``: ``h += delta`` (if given), then
   the normalised rows (all rows, or the rows listed in ``rows``).  ``delta`` is ``[tokens, width]``
   in the activation dtype, or float32 ``[planes, tokens, width]`` whose planes are summed (a
-  mixer or feed-forward may hand on the partial products of its last matrix product).
+  mixer or feed-forward may hand on the partial products of its last matrix product), or a ``Gated``
+  (such a result with the gate it joins the residual behind; the RMS norm takes it).
 * ``Mixer.cache_need() -> KVNeed | StateNeed | None`` and
   ``Mixer.forward(x, step, view) -> delta``; ``view`` is what the cache holds for this place
   in the layer order (``KVView``, ``StateView`` or ``None``).
@@ -89,6 +90,18 @@ class Term:
     y: torch.Tensor
     scale: float = 1.0
     row: torch.Tensor = None
+
+
+@dataclass
+class Gated:
+    """A sublayer's result that joins the residual behind a gate: ``mult * y * sigmoid(z + bias)``, element by
+    element.  y: [tokens, width] in the activation dtype, or float32 planes [planes, tokens, width] that are summed;
+    z: [tokens, width] in the activation dtype; bias: float32 [width] or None.  A norm takes it where it takes a
+    plain delta and does the gating, the add and its own work in one kernel."""
+    y: torch.Tensor
+    z: torch.Tensor
+    bias: torch.Tensor = None
+    mult: float = 1.0
 
 
 class Part:

@@ -45,7 +45,8 @@ class Embedding(Part):
 
 
 class LMHead(Part):
-    """params: vocab, width.  names: weight (the embedding's name when tied)."""
+    """params: vocab, width, softcap (optional; a positive number c: logits <- c * tanh(logits / c)).
+    names: weight (the embedding's name when tied)."""
     graph_safe = True
 
     def tensor_specs(self):
@@ -54,6 +55,7 @@ class LMHead(Part):
     def bind(self, tensors, rt):
         self.rt = rt
         self.weight = rt.weight(tensors[self.names["weight"]])
+        self.softcap = float(self.params.get("softcap") or 0.0)
 
     def step_bytes(self, rows):
         return self.weight.w.numel() * self.weight.w.element_size() if rows else 0
@@ -62,4 +64,5 @@ class LMHead(Part):
         return 2 * rows * self.weight.w.numel()
 
     def forward(self, x):
-        return self.rt.linear(x, self.weight, out_dtype=torch.float32)
+        logits = self.rt.linear(x, self.weight, out_dtype=torch.float32)
+        return self.rt.ops.softcap(logits, self.softcap) if self.softcap > 0 else logits

@@ -6,7 +6,12 @@ A head's plain key is ``W_uk c`` and its value ``W_uv c``; score = (q_plain . k_
 causal softmax, output projection over the concatenated heads.  Only ``[c | k_rot]`` is cached: the scores are
 computed as ``(W_uk^T q_plain) . c`` and the values applied as ``W_uv (sum_j p_j c_j)``, which is the same
 function, so the cache holds one row of kv_rank + rot_dim lanes per token for all heads and no value pages.
-Rotation: lane i of the first ``rot_dims`` turned lanes pairs with lane i + rot_dims/2."""
+Rotation: lane i of the first ``rot_dims`` turned lanes pairs with lane i + rot_dims/2 (``pairing="half"``, the
+default), or lane 2i with lane 2i + 1 (``pairing="adjacent"``).
+
+Variants by parameter: queries through a latent of their own (``q_rank``): ``c_q = rmsnorm(W_dq x)`` with a stored
+weight, ``q = W_uq c_q``; a layer that borrows (``borrows=True``) has no ``W_dkv``: it reads the rows
+``[c | k_rot]`` that an earlier layer keeps, as cached, and expands them with its own ``W_uk`` and ``W_uv``."""
 from __future__ import annotations
 
 import os
@@ -21,15 +26,24 @@ MFMA_MAX_PIECES = 64           # most pieces the matrix-core decode cuts a seque
 
 class LatentAttention(Mixer):
     """params: width, heads, dim, rot_dim, vdim, kv_rank, scale, rot_dims, eps, position (the rotary table's
-    owner, given by the model builder).  names: q, dkv, dkv_norm, uk, uv, o."""
+    owner, given by the model builder), pairing ("half", the default, or "adjacent"), q_rank (0, the default: queries
+    projected directly; else the size of the queries' latent), borrows (default False).
+    names: q (or dq, dq_norm, uq with a query latent), uk, uv, o and, unless the layer borrows, dkv, dkv_norm."""
     graph_safe = True
 
     def tensor_specs(self):
         p, n = self.params, self.names
         d, H, dn, dr, dv, R = p["width"], p["heads"], p["dim"], p["rot_dim"], p["vdim"], p["kv_rank"]
-        return {n["q"]: TensorSpec((H * (dn + dr), d)), n["dkv"]: TensorSpec((R + dr, d)),
-                n["dkv_norm"]: TensorSpec((R,)), n["uk"]: TensorSpec((H * dn, R)), n["uv"]: TensorSpec((H * dv, R)),
-                n["o"]: TensorSpec((d, H * dv))}
+        specs = {n["uk"]: TensorSpec((H * dn, R)), n["uv"]: TensorSpec((H * dv, R)), n["o"]: TensorSpec((d, H * dv))}
+        qr = int(p.get("q_rank", 0))
+        if qr:
+            specs.update({n["dq"]: TensorSpec((qr, d)), n["dq_norm"]: TensorSpec((qr,)),
+                          n["uq"]: TensorSpec((H * (dn + dr), qr))})
+        else:
+            specs[n["q"]] = TensorSpec((H * (dn + dr), d))
+        if not p.get("borrows"):
+            specs.update({n["dkv"]: TensorSpec((R + dr, d)), n["dkv_norm"]: TensorSpec((R,))})
+        return specs
 
     def cache_need(self):
         """One row [latent | turned key part] per token for all heads.  Where the matrix-core attention runs
@@ -47,12 +61,22 @@ class LatentAttention(Mixer):
         if self.rot % 2 or not 0 <= self.rot <= self.dr:
             raise ValueError(f"{self.rot} turning lanes do not fit a turned part of {self.dr} lanes")
         self.position = p["position"]
-        ws = [tensors[n["q"]], tensors[n["dkv"]]]
-        if ws[0].dtype != ws[1].dtype:
+        pairing = p.get("pairing", "half")
+        if pairing not in ("half", "adjacent"):
+            raise ValueError(f"latent attention: pairing={pairing!r} unknown (half, adjacent)")
+        self.adjacent, self.borrows, self.q_rank = pairing == "adjacent", bool(p.get("borrows")), int(p.get("q_rank", 0))
+        ws = [tensors[n["dq"] if self.q_rank else n["q"]]] + ([] if self.borrows else [tensors[n["dkv"]]])
+        if len({w.dtype for w in ws}) != 1:
             ws = [w.float() for w in ws]
         self.n_q = ws[0].shape[0]
+        if len(ws) > 1 and self.n_q % 8:      # the down-projection's columns start at a multiple of eight
+            ws.insert(1, torch.zeros(8 - self.n_q % 8, ws[0].shape[1], dtype=ws[0].dtype, device=ws[0].device))
+        self.down_at = sum(w.shape[0] for w in ws[:-1]) if not self.borrows else 0
         self.w_in = rt.weight(torch.cat(ws, dim=0))
-        self.norm_w = tensors[n["dkv_norm"]].float().contiguous()
+        self.norm_w = None if self.borrows else tensors[n["dkv_norm"]].float().contiguous()
+        if self.q_rank:
+            self.q_norm_w = tensors[n["dq_norm"]].float().contiguous()
+            self.w_uq = rt.weight(tensors[n["uq"]])
         H, dn, dv, R = self.H, self.dn, self.dv, self.R
         self.w_uk_t = tensors[n["uk"]].view(H, dn, R).transpose(1, 2).contiguous()   # [H, R, dn]: q_plain -> latent lanes
         self.w_uv = tensors[n["uv"]].view(H, dv, R).contiguous()
@@ -61,11 +85,14 @@ class LatentAttention(Mixer):
         self.use_mfma = (os.environ.get("BURN_LM_AMD_LATENT_MFMA") != "0" and self.w_uk_t.dtype == torch.bfloat16
                          and rt.ops.latent_attn_mfma_supported(rt.dtype, R, self.dr))
 
+    def _matrices(self):
+        return [self.w_in.w, self.w_o.w, self.w_uk_t, self.w_uv] + ([self.w_uq.w] if self.q_rank else [])
+
     def step_bytes(self, rows):
-        return sum(w.numel() * w.element_size() for w in (self.w_in.w, self.w_o.w, self.w_uk_t, self.w_uv))
+        return sum(w.numel() * w.element_size() for w in self._matrices())
 
     def step_flops(self, rows):
-        return 2 * rows * (self.w_in.w.numel() + self.w_o.w.numel() + self.w_uk_t.numel() + self.w_uv.numel())
+        return 2 * rows * sum(w.numel() for w in self._matrices())
 
     def mixing_flops(self, past, new):
         """Scores over kv_rank + rot_dim lanes and weighted latents over kv_rank lanes, per (query, visible row, head)."""
@@ -81,15 +108,27 @@ class LatentAttention(Mixer):
         rt, ops = self.rt, self.rt.ops
         H, dn, dr, R = self.H, self.dn, self.dr, self.R
         T = x.shape[0]
-        qd = rt.linear(x, self.w_in)                         # [T, H (dn + dr) | R + dr]
-        q, down = qd[:, :self.n_q], qd[:, self.n_q:]
+        if self.borrows == bool(view.store):
+            raise ValueError("a layer with a down-projection keeps its own rows, a borrowing layer reads another's")
+        qd = rt.linear(x, self.w_in)                         # [T, H (dn + dr) or q_rank | R + dr]
+        q, down = qd[:, :self.n_q], (None if self.borrows else qd[:, self.down_at:])
+        if self.q_rank:
+            cq = rt.ops.rmsnorm_rows(q, self.q_norm_w, self.eps, torch.empty(T, self.q_rank, dtype=qd.dtype, device=x.device))
+            q = rt.linear(cq, self.w_uq)
         mfma = self.use_mfma and view.v.numel() > 0 and view.page_size == 64
         qabs = torch.empty(T, H, R + dr, dtype=rt.dtype if mfma else torch.float32, device=x.device)
-        ops.latent_write(down, q, self.norm_w, self.eps, self.position.table, self.rot, qabs, view.k, step,
-                         view.block_table(step), view.page_size, H, dn, R, dr, write_kv=view.store,
-                         vcache=view.v if mfma else None)
+        ops.latent_write(down, q, self.norm_w if self.norm_w is not None else self.q_norm_w_dummy(), self.eps,
+                         self.position.table, self.rot, qabs, view.k, step, view.block_table(step), view.page_size, H, dn,
+                         R, dr, write_kv=view.store, vcache=view.v if mfma and view.store else None,
+                         adjacent=self.adjacent)
         ops.head_project(q, dn + dr, self.w_uk_t, qabs.view(T, H * (R + dr)), R + dr)
         return qabs
+
+    def q_norm_w_dummy(self):
+        """A borrowing layer writes no rows and so has no weight for their norm; the kernel's check wants its size."""
+        if not hasattr(self, "_no_norm"):
+            self._no_norm = torch.ones(self.R, dtype=torch.float32, device=self.rt.device)
+        return self._no_norm
 
     def attend(self, qabs, step, view):
         """Every (token, head)'s weighted sum of the latents it sees -> float32 [tokens, heads, kv_rank]."""

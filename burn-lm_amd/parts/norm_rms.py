@@ -8,20 +8,24 @@ from __future__ import annotations
 
 import torch
 
-from .base import Norm, TensorSpec
+from .base import Gated, Norm, TensorSpec
 
 
 class RMSNorm(Norm):
-    """params: width, eps.  names: weight."""
+    """params: width, eps, single (default False; True: the stored weight is one number for all lanes, a tensor without
+    dimensions).  names: weight."""
     graph_safe = True
 
 
     def tensor_specs(self):
-        return {self.names["weight"]: TensorSpec((self.params["width"],))}
+        return {self.names["weight"]: TensorSpec(() if self.params.get("single") else (self.params["width"],))}
 
     def bind(self, tensors, rt):
         self.rt = rt
-        self.gamma = tensors[self.names["weight"]].contiguous()
+        self.gamma = tensors[self.names["weight"]]
+        if self.params.get("single"):      # the kernels read a weight per lane: the one number, once for each
+            self.gamma = self.gamma.reshape(1).expand(self.params["width"])
+        self.gamma = self.gamma.contiguous()
         self.eps = float(self.params["eps"])
 
     def step_bytes(self, rows):
@@ -33,4 +37,7 @@ class RMSNorm(Norm):
     def add_norm(self, h, delta, rows=None, write_h=True):
         n = h.shape[0] if rows is None else rows.shape[0]
         out = torch.empty(n, h.shape[1], dtype=self.rt.dtype, device=h.device)
+        if isinstance(delta, Gated):
+            return self.rt.ops.add_rmsnorm(h, delta.y, self.gamma, self.eps, out, rows=rows, write_h=write_h,
+                                           gate=delta.z, gate_bias=delta.bias, mult=delta.mult)
         return self.rt.ops.add_rmsnorm(h, delta, self.gamma, self.eps, out, rows=rows, write_h=write_h)

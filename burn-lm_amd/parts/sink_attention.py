@@ -12,7 +12,10 @@ are float32 in every mode.
 
 Variants by parameter: no biases at all (``bias=False``); turning pairs of adjacent lanes ``(2i, 2i + 1)``
 (``pairing="adjacent"``); values that are the keys as projected, before the rotation, with no value projection
-(``values="keys"``; then ``vdim = dim``)."""
+(``values="keys"``; then ``vdim = dim``); a stored temperature per head that multiplies the head's scores
+(``temperature=True``; it rides on the queries, which the scores are linear in, applied in float32 behind their
+rotation); an output gate (``gate=True``): the concatenated heads are multiplied element by element by
+``sigmoid(W_g x)`` of the mixer's own input before the output projection (``W_g`` runs with the other projections)."""
 from __future__ import annotations
 
 import os
@@ -28,9 +31,11 @@ class SinkAttention(Mixer):
     (a rotary encoding whose table has rot_dims/2 pairs; given by the model builder), borrows, sink, talk (whether
     the layer has them; default True), bias (whether the projections have biases; default True), pairing ("half",
     the default: lane i turns with lane i + rot_dims/2; "adjacent": lane 2i with 2i + 1), values ("projected", the
-    default, or "keys": the unrotated keys are the values and there is no value projection).
-    names: q, q_bias, o, o_bias, sink, talk and, unless the layer borrows, k, k_bias, v, v_bias (those the parameters
-    leave)."""
+    default, or "keys": the unrotated keys are the values and there is no value projection), temperature (whether a
+    number per head multiplies its scores; default False), gate (whether the heads pass a sigmoid gate projected from
+    the input; default False).
+    names: q, q_bias, o, o_bias, sink, talk, temp, g and, unless the layer borrows, k, k_bias, v, v_bias (those the
+    parameters leave)."""
     graph_safe = True
 
     def _flags(self):
@@ -57,6 +62,10 @@ class SinkAttention(Mixer):
             specs[n["sink"]] = TensorSpec((H,))
         if talk:
             specs[n["talk"]] = TensorSpec((H, H))
+        if p.get("temperature"):
+            specs[n["temp"]] = TensorSpec((H,))
+        if p.get("gate"):
+            specs[n["g"]] = TensorSpec((H * dv, d))
         if not borrows:
             specs[n["k"]] = TensorSpec((G * dk, d))
             if not values_are_keys:
@@ -83,6 +92,16 @@ class SinkAttention(Mixer):
             raise ValueError("rot_dims must be even, at most the key head size, and come with a rotary encoding")
         roles = ("q",) if self.borrows else ("q", "k") if self.values_are_keys else ("q", "k", "v")
         ws = [tensors[n[r]] for r in roles]
+        self.gated = bool(p.get("gate"))
+        if self.gated and bias:
+            raise ValueError("sink attention: an output gate comes without projection biases")
+        if self.gated:
+            # the gate's columns start at a multiple of eight, so that rows of eight can be read from them at once
+            rows = sum(w.shape[0] for w in ws)
+            if rows % 8:
+                ws.append(torch.zeros(8 - rows % 8, ws[0].shape[1], dtype=ws[0].dtype, device=ws[0].device))
+            self.gate_at = sum(w.shape[0] for w in ws)
+            ws.append(tensors[n["g"]])
         if len({w.dtype for w in ws}) != 1:
             ws = [w.float() for w in ws]
         rows = sum(w.shape[0] for w in ws)
@@ -102,6 +121,7 @@ class SinkAttention(Mixer):
         if self.on_matrix_cores:
             rt.ops.latent_attn_init(rt.device)     # the pieces' workspace, before any step is recorded
             rt.ops.sink_attn_mfma_init(rt.device)  # likewise: the shared memory of the form that stages pages
+        self.temperature = tensors[n["temp"]].float().contiguous() if p.get("temperature") else None
         self.sinks = tensors[n["sink"]].float().contiguous() if sink else None
         self.talk = tensors[n["talk"]].float().contiguous() if talk else None
 
@@ -145,10 +165,19 @@ class SinkAttention(Mixer):
             raise ValueError("a layer with key and value projections keeps its own pages, a borrowing layer reads another's")
         rt.ops.qkv_prepare(qkv, self.bias_in, self.position.table if self.rot else None, self.rot, step,
                            view.block_table(step), view.k, view.v, view.page_size, self.H, self.G, self.dk, self.dv,
-                           write_kv=store, adjacent=self.adjacent, values_are_keys=self.values_are_keys)
+                           write_kv=store, adjacent=self.adjacent, values_are_keys=self.values_are_keys,
+                           q_scale=self.temperature)
         return qkv
 
     def attend(self, qkv, step, view):
+        """What the output projection reads: the heads' results, behind the output gate where the layer has one."""
+        out = self._attend(qkv, step, view)
+        if self.gated:
+            n = self.H * self.dv
+            self.rt.ops.sigmoid_gate(out, qkv[:, self.gate_at:self.gate_at + n])
+        return out
+
+    def _attend(self, qkv, step, view):
         """Every token's queries over its sequence's visible keys -> [tokens, heads * vdim].  bfloat16 with pages of
         64 keys and head sizes the matrix-core kernel takes: that kernel, its pages cut into pieces when a step
         brings so few tiles (decoding) that they would leave most of the chip idle; else the generic kernel."""
