@@ -59,8 +59,9 @@ def attention(W, p, m, h):
     q = (h @ W[p + "q"].T).reshape(T, H, dk)
     k = (h @ W[p + "k"].T).reshape(T, G, dk)
     v = (h @ W[p + "v"].T).reshape(T, G, dv)
-    rot = m["rot"]
-    q, k = turn(q, pos, rot["dims"], rot["base"], "half"), turn(k, pos, rot["dims"], rot["base"], "half")
+    rot = m.get("rot")
+    if rot and rot["dims"]:
+        q, k = turn(q, pos, rot["dims"], rot["base"], "half"), turn(k, pos, rot["dims"], rot["base"], "half")
     scales = m["scale"] * W[p + "temp"].astype(np.float64)
     o = causal_softmax_heads(q, k, v, scales, H // G).reshape(T, H * dv)
     return (o * sigmoid(h @ W[p + "g"].T)) @ W[p + "o"].T
@@ -74,11 +75,12 @@ def lightning(W, p, m, h, eps, state=None):
     q = silu(h @ W[p + "q"].T).reshape(T, H, dk)
     k = silu(h @ W[p + "k"].T).reshape(T, H, dk)
     v = silu(h @ W[p + "v"].T).reshape(T, H, dv)
+    decay = m["decay"] if isinstance(m["decay"], (list, tuple)) else [m["decay"]] * H      # one number: every head's
     S = np.zeros((H, dk, dv)) if state is None else state.copy()
     o = np.zeros((T, H, dv))
     for t in range(T):
         for hd in range(H):
-            S[hd] = m["decay"][hd] * S[hd] + np.outer(k[t, hd], v[t, hd])
+            S[hd] = decay[hd] * S[hd] + np.outer(k[t, hd], v[t, hd])
             o[t, hd] = S[hd].T @ q[t, hd]
     o = rms_norm(o.reshape(T, H * dv), W[p + "norm"], eps) * sigmoid(h @ W[p + "g"].T)
     return o @ W[p + "o"].T, S
