@@ -355,9 +355,34 @@ def girelix_config(width, ff, heads, layers, vocab):
                 layers=[dict(type="parallel", mixer=mixer, mlp=moe) for _ in range(layers)])
 
 
-DESIGNS = {"fuvirax": fuvirax_config, "digasun": digasun_config, "girelix": girelix_config}
+def bitonex_config(width, ff, heads, layers, vocab):
+    """Latent attention (a latent of 512 + 64 lanes, queries through a latent of 768), lightning attention, latent
+    attention that reads the first layer's rows, and two layers of softmax attention (heads of 128 lanes in groups of
+    four, half of each head's lanes turning), in turn; heads of 128 lanes throughout; every layer has the gated dense
+    feed-forward with the Llama's inner size (the same three matrices) and the two gates of the residual."""
+    mlp = dict(kind="dense", ff=8192)
+    lat = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=768, rot=dict(base=500000.0, dims=64),
+               scale=192 ** -0.5)
+    made = []
+    for i in range(layers):
+        k = i % 5
+        if k == 0:
+            made.append(dict(type="latent_attention", mlp=mlp, mixer=dict(lat)))
+        elif k == 1:
+            made.append(dict(type="lightning", mlp=mlp, mixer=dict(
+                heads=heads, dim=128, vdim=128, decay=[1.0 - 2.0 ** -(2 + 6 * h / heads) for h in range(heads)])))
+        elif k == 2:
+            made.append(dict(type="latent_attention", mlp=mlp, mixer=dict(lat, kv_from=i - 2)))
+        else:
+            made.append(dict(type="attention", mlp=mlp, mixer=dict(heads=heads, kv_heads=heads // 4, dim=128, vdim=128,
+                                                                   scale=128 ** -0.5, rot=dict(base=500000.0, dims=64))))
+    return dict(architecture="Bitonex", vocab=vocab, width=width, norm=dict(eps=1e-6), residual_mult=0.7, logit_softcap=30.0,
+                layers=made)
+
+
+DESIGNS = {"fuvirax": fuvirax_config, "digasun": digasun_config, "girelix": girelix_config, "bitonex": bitonex_config}
 # the designs that run beside one (the Llama of equal size always does): the closest of those that were there before
-BESIDE = {"girelix": ("digasun",)}
+BESIDE = {"girelix": ("digasun",), "bitonex": ("girelix", "fuvirax")}
 
 
 def mixer_rates(engine, batch, context, prefill_tokens):
@@ -449,7 +474,7 @@ def mixer_rates(engine, batch, context, prefill_tokens):
 
 
 def run_design(args):
-    """--design fuvirax | digasun | girelix: prompt and decode throughput of the design at sizes that resemble a real
+    """--design fuvirax | digasun | girelix | bitonex: prompt and decode throughput of the design at sizes that resemble a real
     model's layers (random weights), beside the Llama of equal size (and, for a design that has one, the closest earlier
     design), and the mixing kernels of all alone against their limits."""
     import torch
@@ -552,7 +577,7 @@ def main():
                          "launched kernel by kernel on a cache that is filled without a prompt step; prints its time and "
                          "no JSON line, and says on stderr where it is")
     ap.add_argument("--design", default=None, metavar="NAME",
-                    help="instead of the default measurement: prompt and decode throughput of a design (fuvirax, digasun, girelix) at model-like "
+                    help="instead of the default measurement: prompt and decode throughput of a design (fuvirax, digasun, girelix, bitonex) at model-like "
                          "layer sizes beside the Llama of equal size, with the mixing kernels alone (--layers, default 6; "
                          "--sizes 1b-like,3b-like)")
     ap.add_argument("--sizes", default=None, help="with --design: which of its sizes, with commas between them")

@@ -27,6 +27,15 @@ __device__ __forceinline__ uint4 ld16_stream(const bf16* p) { return load16_stre
 
 // KSTEPS: k-steps of 32 per wavefront.  MAXT: most threads of a block (sets the register budget).
 // KEEP_A: the activations' fragments stay in registers across the block's column tiles.
+// the gate branch's activation of a gated product: c_mode 1: silu; c_mode 2: the tanh form of GELU
+__device__ __forceinline__ float gv_gate(float g, int c_mode) {
+  if (c_mode == 2) {
+    const float a = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return 0.5f * g * (2.0f - 2.0f / (1.0f + expf(2.0f * a)));      // 1 + tanh(a) = 2 - 2 / (1 + e^(2a))
+  }
+  return g / (1.0f + expf(-g));
+}
+
 template <int KSTEPS, int MAXT, bool KEEP_A, typename TC>
 __global__ void __launch_bounds__(MAXT)
     gemv_mfma_kernel(const bf16* __restrict__ A, const bf16* __restrict__ Wp, TC* __restrict__ C, int M, int N,
@@ -176,7 +185,7 @@ __global__ void __launch_bounds__(MAXT)
             u += red[w2 * 256 + idx + 8];
           }
           const int nn = tile * 8 + col;
-          if (m < M && nn < N / 2) C[(size_t)m * ldc + nn] = from_float<TC>(g / (1.0f + expf(-g)) * u);
+          if (m < M && nn < N / 2) C[(size_t)m * ldc + nn] = from_float<TC>(gv_gate(g, c_mode) * u);
         }
       }
       __syncthreads();
@@ -277,7 +286,7 @@ __global__ void __launch_bounds__(512)
           u += red[(w2 * MT + mt) * 256 + i + 8];
         }
         const int nn = tile * 8 + col;
-        if (m < M && nn < N / 2) C[(size_t)m * ldc + nn] = from_float<TC>(g / (1.0f + expf(-g)) * u);
+        if (m < M && nn < N / 2) C[(size_t)m * ldc + nn] = from_float<TC>(gv_gate(g, c_mode) * u);
       }
     }
     __syncthreads();
@@ -388,7 +397,7 @@ static int launch_mfma(const void* A, const void* Wp, void* C, int M, int N, int
 }
 
 // Wp: the packed copy of W[N, K] (see the head of this file), ceil(N/16) * ceil(K/32) * 512 elements.
-// c_mode 0: C[M, N] = A W^T.
+// c_mode 0: C[M, N] = A W^T.  (c_mode 2: as c_mode 1 with the tanh form of GELU in place of silu.)
 // c_mode 1: the rows of W come in blocks of 8 gate rows followed by their 8 up rows (so every
 //           16-column tile holds 8 gated pairs) and C[M, N/2] = silu(gate) * up: the SwiGLU gating
 //           fused into the product that feeds it.
@@ -399,7 +408,7 @@ extern "C" int blm_gemv_mfma(const void* A, const void* Wp, void* C, int c_dtype
                              int ldc, int c_mode, int k_groups, hipStream_t stream) {
   BLM_REQUIRE(M >= 1 && M <= 64, "gemv_mfma: M=%d out of range 1..64", M);
   BLM_REQUIRE(N >= 1 && K >= 8 && K % 8 == 0, "gemv_mfma: sizes N=%d K=%d not supported (K a multiple of 8)", N, K);
-  BLM_REQUIRE(c_mode == 0 || (c_mode == 1 && N % 16 == 0 && k_groups == 1),
+  BLM_REQUIRE(c_mode == 0 || ((c_mode == 1 || c_mode == 2) && N % 16 == 0 && k_groups == 1),
               "gemv_mfma: c_mode %d needs N a multiple of 16 and one K group", c_mode);
   BLM_REQUIRE(k_groups >= 1 && k_groups <= 64 && (k_groups == 1 || c_dtype == BLM_F32),
               "gemv_mfma: k_groups=%d needs 1..64 and a float output when above 1", k_groups);

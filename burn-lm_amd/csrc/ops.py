@@ -540,14 +540,16 @@ def pack_weight(w, gated=False):
     return w.view(Np // 16, 16, Kp // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
 
 
-def gemv_mfma(a, packed, out, K, gated=False):
+def gemv_mfma(a, packed, out, K, gated=False, activation="silu"):
     """bfloat16 product for M <= 64 rows on the matrix cores; streams the packed weights once (17 to 64
     rows: K at most 2048 per group, see gemv_mfma_group_limit).
     packed: pack_weight(w) of w [N, K].  out: bfloat16 or float32 [M, N], or float32
     [groups, M, N]: K is then cut into that many groups whose partial products fill the planes of
     out (the reader sums them).  gated=True: packed = pack_weight(w, gated=True) of a [2I, K] matrix
-    and out is [M, I] = silu(a gate^T) * (a up^T)."""
+    and out is [M, I] = act(a gate^T) * (a up^T) with act = silu, or (activation="gelu_tanh") the tanh form of GELU."""
     _gpu(a, packed, out)
+    if activation not in ("silu", "gelu_tanh"):
+        raise KernelError(f"gemv_mfma: activation {activation!r} unknown (silu, gelu_tanh)")
     groups = 1
     if out.dim() == 3:
         groups = out.shape[0]
@@ -565,7 +567,7 @@ def gemv_mfma(a, packed, out, K, gated=False):
     if a.dtype != torch.bfloat16 or packed.dtype != torch.bfloat16:
         raise KernelError("gemv_mfma: operands must be bfloat16")
     _call("blm_gemv_mfma", a.data_ptr(), packed.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0),
-          out.stride(-2), 1 if gated else 0, groups, _stream())
+          out.stride(-2), (2 if activation == "gelu_tanh" else 1) if gated else 0, groups, _stream())
     return out
 
 

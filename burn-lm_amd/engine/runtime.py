@@ -386,13 +386,25 @@ class Runtime:
             return K > 4096 or -(-inner // 32) > 2 * self.compute_units
         return K > 4096 and -(-inner // 32) > self.compute_units
 
-    def gated_linear(self, x, w):
-        """silu(x gate^T) * (x up^T) for w = [gate rows; up rows] ([2I, K]) -> [M, I].  With few rows
-        in bfloat16 the gating is fused into the product (weight(w, gated=True) pairs the rows for
-        it); otherwise the product is followed by the gating kernel."""
+    def gated_linear(self, x, w, activation="silu"):
+        """act(x gate^T) * (x up^T) for w = [gate rows; up rows] ([2I, K]) -> [M, I]; act is silu or
+        (activation="gelu_tanh") the tanh form of GELU.  With few rows in bfloat16 the gating is fused
+        into the product (weight(w, gated=True) pairs the rows for it); otherwise the product is followed
+        by the gating kernel."""
         M, K = x.shape
         inner = w.shape[0] // 2
         plain = w.w if isinstance(w, LinearWeight) else w
+        if activation != "silu":
+            if activation != "gelu_tanh":
+                raise ValueError(f"gated_linear: activation {activation!r} unknown (silu, gelu_tanh)")
+            # the packed skinny product takes the activation; the kernels for more rows gate with silu only
+            if (isinstance(w, LinearWeight) and w.packable and w.gated and x.dtype == torch.bfloat16
+                    and M <= self.skinny_gated_rows and ops.gemv_mfma_supported(M, w.shape[0], K)
+                    and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+                out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
+                return ops.gemv_mfma(x, w.packed, out, K, gated=True, activation=activation)
+            gu = self.linear(x, plain)
+            return ops.gelu_glu(gu, torch.empty(M, inner, dtype=gu.dtype, device=x.device))
         fusable = (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(1) == 1
                    and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and plain.is_contiguous())
         by_library = 16 < M <= MFMA_SKINNY_MAX_ROWS and self._gated_by_library(M, K, inner)

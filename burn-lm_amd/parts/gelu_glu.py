@@ -1,6 +1,7 @@
 """Dense gated feed-forward with the tanh form of GELU: ``W_down (gelu_tanh(W_gate x) * (W_up x))`` without biases,
 ``gelu_tanh(z) = z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``.  Gate and up run as one product on the stacked
-weight; the activation and the product are float32 in a kernel of their own."""
+weight; the activation and the product are float32, in the product's own epilogue when few rows run (decode) and in
+a kernel of their own otherwise."""
 from __future__ import annotations
 
 import torch
@@ -22,7 +23,7 @@ class GeluGLU(FeedForward):
         g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.w_gate_up = rt.weight(torch.cat([g, u], dim=0))
+        self.w_gate_up = rt.weight(torch.cat([g, u], dim=0), gated=True)
         self.w_down = rt.weight(tensors[self.names["down"]])
         self.inner = self.params["inner"]
 
@@ -34,6 +35,4 @@ class GeluGLU(FeedForward):
 
     def forward(self, x, step):
         rt = self.rt
-        gu = rt.linear(x, self.w_gate_up)
-        act = torch.empty(x.shape[0], self.inner, dtype=gu.dtype, device=x.device)
-        return rt.linear(rt.ops.gelu_glu(gu, act), self.w_down, partials=True)
+        return rt.linear(rt.gated_linear(x, self.w_gate_up, activation="gelu_tanh"), self.w_down, partials=True)
