@@ -135,20 +135,27 @@ class BitonexConfig:
                 mixer = LightningConfig(heads=heads, dim=_get(m, "dim", int, mw), vdim=_get(m, "vdim", int, mw),
                                         decay=tuple(float(a) for a in decay))
             elif kind == "latent_attention":
-                rot_dim = _get(m, "rot_dim", int, mw)
-                rot_dims, rot_base = _rot(m, mw, rot_dim)
-                kv_from = m.get("kv_from")
+                kv_from = m.get("kv_from") if isinstance(m, dict) else None
+                src = None
                 if kv_from is not None:
                     if isinstance(kv_from, bool) or not isinstance(kv_from, int) or not 0 <= kv_from < i:
                         raise ConfigError(f"config.json: {mw}.kv_from must name an earlier layer, got {kv_from!r}")
                     src = out[kv_from].mixer
                     if src.type != "latent_attention" or src.kv_from is not None:
                         raise ConfigError(f"config.json: {mw}.kv_from names layer {kv_from}, which keeps no latent rows of its own")
+                    # what the rows' shape decides may be left to the layer that keeps them
+                    m = dict(m)
+                    m.setdefault("kv_rank", src.kv_rank)
+                    m.setdefault("rot_dim", src.rot_dim)
+                    if m.get("rot") is None and src.rot_dims:
+                        m["rot"] = dict(dims=src.rot_dims, base=src.rot_base)
+                rot_dim = _get(m, "rot_dim", int, mw)
+                rot_dims, rot_base = _rot(m, mw, rot_dim)
                 mixer = LatentConfig(heads=_get(m, "heads", int, mw), dim=_get(m, "dim", int, mw), rot_dim=rot_dim,
                                      vdim=_get(m, "vdim", int, mw), kv_rank=_get(m, "kv_rank", int, mw),
                                      q_rank=_get(m, "q_rank", int, mw) if m.get("q_rank") is not None else None,
                                      scale=_get(m, "scale", float, mw), rot_dims=rot_dims, rot_base=rot_base, kv_from=kv_from)
-                if kv_from is not None and (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != \
+                if src is not None and (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != \
                         (mixer.kv_rank, mixer.rot_dim, mixer.rot_dims, mixer.rot_base):
                     raise ConfigError(f"config.json: {mw} reads layer {kv_from}'s rows but differs from it in kv_rank, "
                                       f"rot_dim or rotation")

@@ -290,9 +290,11 @@ def whole(eng, toks):
                                     [lightning(mlp=None)], [lightning(heads=1, dim=70, vdim=5, decay=(0.99,), mlp=None)],
                                     [latent(mlp=None)], [latent(heads=4, dim=16, rot_dim=16, vdim=16, kv_rank=32, q_rank=8, mlp=None)],
                                     [latent(mlp=None), latent(heads=2, dim=4, vdim=6, q_rank=16, kv_from=0, mlp=None)],
+                                    [latent(kv_rank=32, rot_dim=16, mlp=None), lightning(mlp=None),
+                                     latent(heads=18, dim=4, vdim=6, kv_rank=32, rot_dim=16, q_rank=16, kv_from=0, mlp=None)],
                                     [lightning(heads=1, dim=8, vdim=8, decay=(0.5,))]],
                          ids=["attention", "attention_ungrouped", "attention_one_kv_head", "attention_wide_values",
-                              "lightning", "lightning_one_wide_head", "latent", "latent_larger", "latent_read_by_another",
+                              "lightning", "lightning_one_wide_head", "latent", "latent_larger", "latent_read_by_another", "latent_of_a_matrix_core_size_read_by_another",
                               "feed_forward"])
 def test_every_mechanism_alone(tmp_path, layers, dtype):
     cfg = config(layers)
@@ -429,7 +431,9 @@ def test_one_key_far_back_among_hundreds(tmp_path, kind, dtype):
     if kind == "attention":
         cfg = config([attention(heads=4, kv_heads=2, dim=16, vdim=16, rot=8, scale=0.25, mlp=None)], cap=None)
     else:
-        cfg = config([latent(scale=0.25, mlp=None), latent(heads=2, dim=4, vdim=6, q_rank=16, scale=0.25, kv_from=0, mlp=None)], cap=None)
+        # a latent of a size that the matrix-core kernel takes in bfloat16 runs (float32 runs take the generic one)
+        cfg = config([latent(kv_rank=32, rot_dim=16, scale=0.25, mlp=None),
+                      latent(heads=2, dim=4, vdim=6, kv_rank=32, rot_dim=16, q_rank=16, scale=0.25, kv_from=0, mlp=None)], cap=None)
     marker = 7
     w = marked(kind, cfg, make_weights(cfg, 9), marker)
     eng = engine_for(tmp_path, cfg, w, dtype, max_tokens=1024)
