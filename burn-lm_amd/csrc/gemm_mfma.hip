@@ -43,6 +43,14 @@ __device__ __forceinline__ float gm_silu(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
 }
 
+// the tanh form of GELU, z/2 (1 + tanh(a)) with a = sqrt(2/pi) (z + 0.044715 z^3): (1 + tanh(a)) / 2 = sigmoid(2a)
+__device__ __forceinline__ float gm_gelu(float x) {
+  const float a = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a * -2.8853900817779268f));
+}
+template <int MODE>
+__device__ __forceinline__ float gm_gate(float x) { return MODE == 2 ? gm_gelu(x) : gm_silu(x); }
+
 // columns per pass of the epilogue: as many of a wavefront's `on` as the staging of all `waves` leaves room for
 constexpr int gm_pass_columns(int on, int waves, size_t bytes) {
   int cw = on;
@@ -83,7 +91,7 @@ __global__ void __launch_bounds__(WGM* WGN* BLM_WAVE)
   if (total % 8 == 0) t = (t & 7) * (total >> 3) + (t >> 3);
   const int tm = t % m_tiles, tn = t / m_tiles;
   const int m0 = tm * BM;
-  const int n0 = tn * (MODE == 1 ? BN / 2 : BN);   // first output column
+  const int n0 = tn * (MODE != 0 ? BN / 2 : BN);   // first output column
   const int k_begin = blockIdx.y * k_per_group, k_end = min(K, k_begin + k_per_group);
   C += (size_t)blockIdx.y * M * ldc;
 
@@ -109,7 +117,7 @@ __global__ void __launch_bounds__(WGM* WGN* BLM_WAVE)
     const int r = (wave * B_LD + i) * RPL + st_row;
     const int piece = st_slot ^ ((r / RPB) % P);
     int n;   // row of W relative to n0
-    if (MODE == 1) n = r < BN / 2 ? min(r, N - 1 - n0) : N + min(r - BN / 2, N - 1 - n0);
+    if (MODE != 0) n = r < BN / 2 ? min(r, N - 1 - n0) : N + min(r - BN / 2, N - 1 - n0);
     else n = min(r, N - 1 - n0);
     b_off[i] = (uint32_t)(n * ldw + piece * 8) * 2u;
   }
@@ -165,7 +173,7 @@ __global__ void __launch_bounds__(WGM* WGN* BLM_WAVE)
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     int r;
-    if (MODE == 1) r = (j < TN / 2 ? 0 : BN / 2) + wn * (WN / 2) + (j % (TN / 2)) * 32;
+    if (MODE != 0) r = (j < TN / 2 ? 0 : BN / 2) + wn * (WN / 2) + (j % (TN / 2)) * 32;
     else r = wn * WN + j * 32;
     b_row[j] = (r + l32) * BK;
   }
@@ -262,7 +270,7 @@ __global__ void __launch_bounds__(WGM* WGN* BLM_WAVE)
   // Results leave through shared memory, 32 rows and CW columns at a time per wavefront, so that
   // every store writes 16 bytes per lane and runs of whole lines per row.
   __syncthreads();
-  constexpr int ON = MODE == 1 ? WN / 2 : WN;           // output columns of a wavefront
+  constexpr int ON = MODE != 0 ? WN / 2 : WN;           // output columns of a wavefront
   constexpr int CW = gm_pass_columns(ON, NW, (size_t)NS * (BM + BN) * BK * sizeof(bf16));
   static_assert(CW >= 32, "output staging fits");
   constexpr int OSTR = CW + 4;                          // floats per staged row
@@ -279,11 +287,11 @@ __global__ void __launch_bounds__(WGM* WGN* BLM_WAVE)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           float4 v;
-          if (MODE == 1) {
+          if (MODE != 0) {
             float4 gt = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
             float4 up = make_float4(acc[i][j + TN / 2][4 * g], acc[i][j + TN / 2][4 * g + 1],
                                     acc[i][j + TN / 2][4 * g + 2], acc[i][j + TN / 2][4 * g + 3]);
-            v = make_float4(gm_silu(gt.x) * up.x, gm_silu(gt.y) * up.y, gm_silu(gt.z) * up.z, gm_silu(gt.w) * up.w);
+            v = make_float4(gm_gate<MODE>(gt.x) * up.x, gm_gate<MODE>(gt.y) * up.y, gm_gate<MODE>(gt.z) * up.z, gm_gate<MODE>(gt.w) * up.w);
           } else {
             v = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
           }
@@ -349,7 +357,7 @@ static int launch_gemm(const void* A, const void* W, void* C, int M, int N, int 
                        int k_groups, hipStream_t stream) {
   constexpr size_t smem = (size_t)NS * (BM + BN) * BK * sizeof(bf16);
   const int m_tiles = (M + BM - 1) / BM;
-  const int n_tiles = (N + (MODE == 1 ? BN / 2 : BN) - 1) / (MODE == 1 ? BN / 2 : BN);
+  const int n_tiles = (N + (MODE != 0 ? BN / 2 : BN) - 1) / (MODE != 0 ? BN / 2 : BN);
   const int k_per_group = ((K + k_groups - 1) / k_groups + BK - 1) / BK * BK;
   dim3 grid((unsigned)(m_tiles * n_tiles), (unsigned)k_groups), block(WGM * WGN * BLM_WAVE);
   hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, BK, NS, WGM, WGN, MODE, TC>), grid, block, smem, stream, (const bf16*)A,
@@ -365,7 +373,8 @@ static int launch_gemm(const void* A, const void* W, void* C, int M, int N, int 
 extern "C" int blm_gemm_mfma_init() {
 #define BLM_PREP(BM, BN, BK, NS, WGM, WGN)                                                                     \
   if (prepare_gemm<BM, BN, BK, NS, WGM, WGN, 0, bf16>() || prepare_gemm<BM, BN, BK, NS, WGM, WGN, 0, float>() ||       \
-      prepare_gemm<BM, BN, BK, NS, WGM, WGN, 1, bf16>() || prepare_gemm<BM, BN, BK, NS, WGM, WGN, 1, float>())         \
+      prepare_gemm<BM, BN, BK, NS, WGM, WGN, 1, bf16>() || prepare_gemm<BM, BN, BK, NS, WGM, WGN, 1, float>() ||       \
+      prepare_gemm<BM, BN, BK, NS, WGM, WGN, 2, bf16>() || prepare_gemm<BM, BN, BK, NS, WGM, WGN, 2, float>())         \
     return 1;
   BLM_GEMM_TILES(BLM_PREP)
 #undef BLM_PREP
@@ -384,6 +393,7 @@ extern "C" int blm_gemm_mfma_init() {
 // stages of 32 in deeper rings were not faster.  Measured at 256 to 4,096 rows: the largest tile
 // that still gives every compute unit a block is the fastest.
 // mode 0: C[M, N] = A W^T, W [N, K].  mode 1: W [2N, K] = [gate rows; up rows], C[M, N] = silu(gate) * up.
+// mode 2: as mode 1 with the tanh form of GELU in place of silu.
 extern "C" int blm_gemm_mfma(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda,
                              int ldw, int ldc, int mode, int k_groups, int tile, hipStream_t stream) {
   BLM_REQUIRE(M >= 1 && N >= 1 && K >= 8 && K % 8 == 0, "gemm_mfma: sizes M=%d N=%d K=%d not supported (K a multiple of 8)",
@@ -391,15 +401,19 @@ extern "C" int blm_gemm_mfma(const void* A, const void* W, void* C, int c_dtype,
   BLM_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= N, "gemm_mfma: bad strides lda=%d ldw=%d ldc=%d",
               lda, ldw, ldc);
   BLM_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_mfma: operands must be 16-byte aligned");
-  BLM_REQUIRE(mode == 0 || (mode == 1 && k_groups == 1), "gemm_mfma: mode %d needs one K group", mode);
+  BLM_REQUIRE(mode == 0 || ((mode == 1 || mode == 2) && k_groups == 1), "gemm_mfma: mode %d needs one K group", mode);
   BLM_REQUIRE(k_groups >= 1 && k_groups <= 64 && (k_groups == 1 || c_dtype == BLM_F32),
               "gemm_mfma: k_groups=%d needs 1..64 and a float output when above 1", k_groups);
   BLM_REQUIRE(c_dtype == BLM_BF16 || c_dtype == BLM_F32, "gemm_mfma: unsupported output dtype %d", c_dtype);
   // per-lane byte offsets into a tile's rows are 32-bit
-  BLM_REQUIRE((size_t)256 * lda * 2 < ((size_t)1 << 32) && (size_t)(mode == 1 ? 2 : 1) * N * ldw * 2 < ((size_t)1 << 32),
+  BLM_REQUIRE((size_t)256 * lda * 2 < ((size_t)1 << 32) && (size_t)(mode != 0 ? 2 : 1) * N * ldw * 2 < ((size_t)1 << 32),
               "gemm_mfma: matrices of 4 GiB and more are not supported (lda=%d, N=%d, ldw=%d)", lda, N, ldw);
 #define BLM_GEMM(BM, BN, BK, NS, WGM, WGN)                                                                           \
   do {                                                                                                               \
+    if (mode == 2)                                                                                                   \
+      return c_dtype == BLM_BF16                                                                                     \
+                 ? launch_gemm<BM, BN, BK, NS, WGM, WGN, 2, bf16>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream) \
+                 : launch_gemm<BM, BN, BK, NS, WGM, WGN, 2, float>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream); \
     if (mode == 1)                                                                                                   \
       return c_dtype == BLM_BF16                                                                                     \
                  ? launch_gemm<BM, BN, BK, NS, WGM, WGN, 1, bf16>(A, W, C, M, N, K, lda, ldw, ldc, k_groups, stream) \

@@ -614,11 +614,12 @@ def static_scratch_init(device=None):
         _static_ready.add(index)
 
 
-def gemm_mfma(a, w, out, gated=False, tile=(128, 128)):
+def gemm_mfma(a, w, out, gated=False, tile=(128, 128), activation="silu"):
     """bfloat16 product for many rows on the matrix cores: out = a[M, K] @ w[N, K]^T, with w as the
     checkpoint stores it.  out: bfloat16 or float32 [M, N], or float32 [groups, M, N] partial
     products over that many groups of K (the reader sums them).  gated=True: w is [gate rows; up
-    rows] ([2I, K]) and out is [M, I] = silu(a gate^T) * (a up^T).  tile: rows x columns of out (of
+    rows] ([2I, K]) and out is [M, I] = act(a gate^T) * (a up^T), act = silu or (activation="gelu_tanh") the tanh form
+    of GELU.  tile: rows x columns of out (of
     gate and up columns together when gated) per block, one of GEMM_TILES; a third number is the depth of
     the ring of K stages (deep rings for products of few tiles, which wait for memory, not for the matrix cores)."""
     _gpu(a, w, out)
@@ -639,7 +640,7 @@ def gemm_mfma(a, w, out, gated=False, tile=(128, 128)):
     if tile not in GEMM_TILES:
         raise KernelError(f"gemm_mfma: tile {tile} is not one of {sorted(GEMM_TILES)}")
     _call("blm_gemm_mfma", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), M, N, K, a.stride(0), w.stride(0),
-          out.stride(-2), 1 if gated else 0, groups, GEMM_TILES[tile], _stream())
+          out.stride(-2), (2 if activation == "gelu_tanh" else 1) if gated else 0, groups, GEMM_TILES[tile], _stream())
     return out
 
 

@@ -394,21 +394,13 @@ class Runtime:
         M, K = x.shape
         inner = w.shape[0] // 2
         plain = w.w if isinstance(w, LinearWeight) else w
-        if activation != "silu":
-            if activation != "gelu_tanh":
-                raise ValueError(f"gated_linear: activation {activation!r} unknown (silu, gelu_tanh)")
-            # the packed skinny product takes the activation; the kernels for more rows gate with silu only
-            if (isinstance(w, LinearWeight) and w.packable and w.gated and x.dtype == torch.bfloat16
-                    and M <= self.skinny_gated_rows and ops.gemv_mfma_supported(M, w.shape[0], K)
-                    and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
-                out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
-                return ops.gemv_mfma(x, w.packed, out, K, gated=True, activation=activation)
-            gu = self.linear(x, plain)
-            return ops.gelu_glu(gu, torch.empty(M, inner, dtype=gu.dtype, device=x.device))
+        if activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"gated_linear: activation {activation!r} unknown (silu, gelu_tanh)")
+        silu = activation == "silu"      # the row-ring kernel gates with silu only; the others take the activation
         fusable = (x.dtype == plain.dtype == self.dtype == torch.bfloat16 and K % 8 == 0 and x.stride(1) == 1
                    and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and plain.is_contiguous())
         by_library = 16 < M <= MFMA_SKINNY_MAX_ROWS and self._gated_by_library(M, K, inner)
-        if fusable and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and not by_library and (
+        if fusable and silu and self.rows_ring and 16 < M <= MFMA_SKINNY_MAX_ROWS and not by_library and (
                 M > 32 or -(-inner // 32) <= self.compute_units * (2 if K <= RING_GROUP_K else 1)):
             # 33 to 64 rows (measured against the packed skinny kernel: 4-15 % faster at the 1B and 3B shapes, and
             # at wider ones in place of the library's product, which the packed kernel's registers leave them to);
@@ -420,7 +412,7 @@ class Runtime:
                 and M <= self.skinny_gated_rows and ops.gemv_mfma_supported(M, w.shape[0], K)
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
             out = torch.empty(M, inner, dtype=self.dtype, device=x.device)
-            return ops.gemv_mfma(x, w.packed, out, K, gated=True)
+            return ops.gemv_mfma(x, w.packed, out, K, gated=True, activation=activation)
         if fusable and self.fused_gate_up_measured and M > MFMA_SKINNY_MAX_ROWS:
             # Short prompts: when all tiles of the product run at once (one block per compute unit,
             # most of the units busy), the fused kernel with a deep ring of stages streams the
@@ -432,7 +424,7 @@ class Runtime:
                 blocks = m128 * -(-inner // pairs)
                 if self.compute_units // 4 <= blocks <= self.compute_units:
                     return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
-                                         gated=True, tile=tile)
+                                         gated=True, tile=tile, activation=activation)
             # 256x128 tiles that make one round on at least three quarters of the compute units, with rows
             # that fill their tiles to 85 % and more: measured against the library's product and the gating
             # kernel 11-16 % faster with a full round (512 rows of an inner size of 8192 at widths 2048 and
@@ -443,7 +435,7 @@ class Runtime:
             blocks = m256 * -(-inner // 64)
             if M > 256 and M * 20 >= m256 * 256 * 17 and self.compute_units * 3 // 4 <= blocks <= self.compute_units:
                 return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
-                                     gated=True, tile=(256, 128))
+                                     gated=True, tile=(256, 128), activation=activation)
             # Long prompts: with whole rounds of 256x256 tiles (as many blocks as compute units, or a
             # multiple) and a narrow model the fused kernel is ahead of the library over the whole
             # prefill (width 2048: 2-4 % at 1,024 and 2,048 rows, 0.5-0.8 % at 3,072 and 4,096; behind by
@@ -452,14 +444,14 @@ class Runtime:
             # against 20.7, of 16,384 tokens 47.9 against 49.0).
             if K <= RING_GROUP_K and 256 <= M <= 4096 and (-(-M // 256) * -(-inner // 128)) % self.compute_units == 0:
                 return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device),
-                                     gated=True, tile=(256, 256))
+                                     gated=True, tile=(256, 256), activation=activation)
         if fusable and self.fused_gate_up_rows[0] <= M <= self.fused_gate_up_rows[1]:
             # the largest tile that still gives every compute unit a block (a tile of n columns holds n / 2 gated pairs)
             m256 = -(-M // 256)
             tile = ((256, 256) if m256 * -(-inner // 128) >= self.compute_units else
                     (256, 128) if m256 * -(-inner // 64) >= self.compute_units else (128, 128))
-            return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device), gated=True, tile=tile)
+            return ops.gemm_mfma(x, plain, torch.empty(M, inner, dtype=self.dtype, device=x.device), gated=True, tile=tile, activation=activation)
         gu = self.linear(x, plain)
         act = torch.empty(M, inner, dtype=gu.dtype, device=x.device)
-        ops.swiglu(gu, act)
+        (ops.swiglu if silu else ops.gelu_glu)(gu, act)
         return act

@@ -1,7 +1,7 @@
 """Dense gated feed-forward with the tanh form of GELU: ``W_down (gelu_tanh(W_gate x) * (W_up x))`` without biases,
 ``gelu_tanh(z) = z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``.  Gate and up run as one product on the stacked
-weight; the activation and the product are float32, in the product's own epilogue when few rows run (decode) and in
-a kernel of their own otherwise."""
+weight; the activation and the product are float32, in the epilogue of the hand-written products (few rows, and
+prompts of the sizes the runtime gives to its tiled kernel) and in a kernel of their own behind the library's product."""
 from __future__ import annotations
 
 import torch

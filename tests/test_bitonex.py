@@ -698,6 +698,12 @@ def test_gated_add_activation_and_cap_against_the_plain_functions(dtype):
             got = ops.gemv_mfma(x, ops.pack_weight(wgu, gated=True), torch.empty(M, I, dtype=dtype, device=dev), K, gated=True,
                                 activation="gelu_tanh")
             assert rel_err(got.double().cpu().numpy(), P.gelu_tanh(pre[:, :I]) * pre[:, I:]) < tol, (M, K, I)
+        # many rows: the activation in the epilogue of the tiled product
+        for M, K, I, tile in ((130, 128, 192, (128, 128)), (300, 256, 256, (256, 128)), (70, 64, 40, (128, 64, 6))):
+            x, wgu = act(rng.standard_normal((M, K))), act(rng.standard_normal((2 * I, K)) / math.sqrt(K) * 3)
+            pre = x.double().cpu().numpy() @ wgu.double().cpu().numpy().T
+            got = ops.gemm_mfma(x, wgu, torch.empty(M, I, dtype=dtype, device=dev), gated=True, tile=tile, activation="gelu_tanh")
+            assert rel_err(got.double().cpu().numpy(), P.gelu_tanh(pre[:, :I]) * pre[:, I:]) < tol, (M, K, I)
     z = f32(rng.standard_normal((9, 77)) * 40)
     want = 15.0 * np.tanh(z.double().cpu().numpy() / 15.0)
     assert np.abs(ops.softcap(z, 15.0).double().cpu().numpy() - want).max() < 1e-5
