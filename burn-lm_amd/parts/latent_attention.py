@@ -73,7 +73,9 @@ class LatentAttention(Mixer):
             ws.insert(1, torch.zeros(8 - self.n_q % 8, ws[0].shape[1], dtype=ws[0].dtype, device=ws[0].device))
         self.down_at = sum(w.shape[0] for w in ws[:-1]) if not self.borrows else 0
         self.w_in = rt.weight(torch.cat(ws, dim=0))
-        self.norm_w = None if self.borrows else tensors[n["dkv_norm"]].float().contiguous()
+        # (a reading layer writes no rows and has no weight for their norm; the kernel's check wants one of its size)
+        self.norm_w = torch.ones(self.R, dtype=torch.float32, device=rt.device) if self.borrows \
+            else tensors[n["dkv_norm"]].float().contiguous()
         if self.q_rank:
             self.q_norm_w = tensors[n["dq_norm"]].float().contiguous()
             self.w_uq = rt.weight(tensors[n["uq"]])
@@ -117,18 +119,12 @@ class LatentAttention(Mixer):
             q = rt.linear(cq, self.w_uq)
         mfma = self.use_mfma and view.v.numel() > 0 and view.page_size == 64
         qabs = torch.empty(T, H, R + dr, dtype=rt.dtype if mfma else torch.float32, device=x.device)
-        ops.latent_write(down, q, self.norm_w if self.norm_w is not None else self.q_norm_w_dummy(), self.eps,
+        ops.latent_write(down, q, self.norm_w, self.eps,
                          self.position.table, self.rot, qabs, view.k, step, view.block_table(step), view.page_size, H, dn,
                          R, dr, write_kv=view.store, vcache=view.v if mfma and view.store else None,
                          adjacent=self.adjacent)
         ops.head_project(q, dn + dr, self.w_uk_t, qabs.view(T, H * (R + dr)), R + dr)
         return qabs
-
-    def q_norm_w_dummy(self):
-        """A borrowing layer writes no rows and so has no weight for their norm; the kernel's check wants its size."""
-        if not hasattr(self, "_no_norm"):
-            self._no_norm = torch.ones(self.R, dtype=torch.float32, device=self.rt.device)
-        return self._no_norm
 
     def attend(self, qabs, step, view):
         """Every (token, head)'s weighted sum of the latents it sees -> float32 [tokens, heads, kv_rank]."""
